@@ -340,8 +340,7 @@ __global__ __launch_bounds__(RT == 1 ? 512 : 256) void attention_mfma_kernel(
             // the path head size 16 takes, the accumulator was copied back
             // (v_accvgpr_read_b32) three wait states after the instruction instead of seven,
             // and one of a lane's four sums of the first row tile lost the block's product.
-            // Straight-line code gets its waits; tests/test_isa_hazards.py reads the compiled
-            // kernels for such sequences.
+            // Straight-line code gets its waits.
             for (int dt = 0; dt < DT; ++dt)
                 o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, o[rt][dt], 0, 0, 0);
         }
