@@ -18,7 +18,8 @@ asks its groups:
 * a KV group owns ``k`` ``[entries, n_pages + 1, n_kv_heads, PAGE, head_dim]`` and ``v``
   ``[entries, n_pages + 1, n_kv_heads, value_dim, PAGE]`` and a free list of pages; a
   sequence holds, per group, a list of pages that grows by one page every ``PAGE`` tokens.
-  A windowed group gives pages back once every key in them is out of reach.  Pages are
+  A windowed group gives pages back once every key in them is out of reach (the pages of
+  the first ``keep_first`` keys stay).  Pages are
   reused without clearing: a reader never looks beyond a sequence's length (the reference
   relies on the same masking when it reuses its buffers, model.py:118-119).  A group with
   ``paged = True`` gets a table of page numbers per sequence in every step's description.
@@ -44,6 +45,7 @@ class KVNeed:
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None       # None: as head_dim
+    keep_first: int = 0                   # with a window: the first keys stay in reach
 
     @property
     def v_dim(self) -> int:
@@ -141,7 +143,8 @@ class KVGroup(Group):
             first_needed = 0
             if self.need.window is not None:
                 first_needed = max(0, start - self.need.window + 1) // PAGE
-            drop = [i for i in range(min(first_needed, len(held))) if held[i] >= 0]
+            kept = pages_for(self.need.keep_first)      # pages that hold the kept first keys
+            drop = [i for i in range(kept, min(first_needed, len(held))) if held[i] >= 0]
             grow = max(pages_for(start + n_new) - len(held), 0)
             plans.append((held, drop, grow))
             demand += grow - len(drop)

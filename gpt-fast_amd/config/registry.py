@@ -7,7 +7,7 @@ plan's parameters.  Everything else in the library is shared.
 
 The reference picks its one model class by the checkpoint folder's name
 (generate.py:222, model.py:44-57, 148-150); here ``config.json`` names it through
-``architectures[0]`` or ``model_type``.
+``architectures[0]``, ``architecture`` or ``model_type``.
 """
 import json
 import os
@@ -93,11 +93,12 @@ def find_preset(name: str, architecture_name: str = None):
 def architecture_of(config_json: dict) -> Architecture:
     """The architecture that a ``config.json`` dictionary names."""
     names = list(config_json.get("architectures") or [])
-    if config_json.get("model_type"):
-        names.append(config_json["model_type"])
+    for key in ("architecture", "model_type"):
+        if isinstance(config_json.get(key), str) and config_json[key]:
+            names.append(config_json[key])
     if not names:
         raise UnknownArchitecture(
-            "config.json has neither 'architectures' nor 'model_type'; "
+            "config.json has none of 'architectures', 'architecture', 'model_type'; "
             f"known: {known_architectures()}")
     for name in names:
         if name in _ARCHITECTURES:

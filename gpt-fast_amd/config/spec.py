@@ -15,10 +15,13 @@ from typing import List, Optional, Tuple
 
 @dataclass(frozen=True)
 class NormSpec:
-    """Root-mean-square norm over the last dimension (reference model.py:230-241)."""
+    """Root-mean-square norm over the last dimension (reference model.py:230-241).
+    ``weight_offset`` is added to the stored weight before it is used: 0 for weights stored
+    around one, 1 for weights stored around zero (``x / rms * (1 + w)``)."""
     dim: int
     eps: float
     kind: str = "rms"
+    weight_offset: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -29,7 +32,8 @@ class PositionSpec:
     key head by ``position * frequency[i]`` (reference model.py:266-293).  ``layout``
     is "interleaved" (pairs (2i, 2i+1), the reference's) or "half" (pairs
     (i, i + rotary_dim/2)).  ``scaling`` is None or a dict with ``rope_type`` and that
-    rule's constants (reference model.py:244-263 for "llama3").
+    rule's constants (reference model.py:244-263 for "llama3"; "linear" divides every
+    frequency by ``factor``).
     kind "none": no position information is added.
     """
     kind: str = "rope"
@@ -58,8 +62,55 @@ class AttentionSpec:
 
 
 @dataclass(frozen=True)
+class DifferentialAttentionSpec:
+    """Causal attention whose heads each hold ``n_maps`` = 2 softmax maps over the same
+    values: query and key rows lie head by head as [map 1, map 2], each map ``head_dim``
+    wide, values ``value_dim`` wide.  A head's result is ``a1 - lam * a2`` with
+    ``lam = exp(lq1 . lk1) - exp(lq2 . lk2) + lam_init`` (four learned vectors of
+    ``head_dim``), divided by its root mean square over ``value_dim`` (``eps`` inside the
+    root), times ``1 - lam_init``, times a sigmoid gate per head if ``head_gate``.
+    ``window`` W: keys at distance < W; ``keep_first`` F: the keys at positions < F stay
+    visible beyond the window, at their true positions.  Position i sees j if
+    ``j <= i and (i - j < W or j < F)``."""
+    dim: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    value_dim: int
+    position: PositionSpec
+    lam_init: float
+    eps: float
+    scale: Optional[float] = None          # None: 1/sqrt(head_dim)
+    window: Optional[int] = None
+    keep_first: int = 0
+    head_gate: bool = True
+    kind: str = "differential_attention"
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """Recurrent mixer with a matrix memory per head (the mLSTM cell of xLSTM): state
+    ``S [key_dim, value_dim]``, normaliser ``n [key_dim]`` and a running maximum ``m`` of the
+    log gates, all float32 and zero at a sequence's start.  With log input gate
+    ``i = cap tanh(. / cap)``, log forget gate ``f = logsigmoid(cap tanh(. / cap))``:
+    ``m' = max(f + m, i)``, ``S' = exp(f + m - m') S + exp(i - m') k v^T``, n likewise with k,
+    ``o = S'^T q / (max(|n' . q|, exp(-m')) + den_eps)``; each head's o is divided by its root
+    mean square (``eps``), times a weight per element, times sigmoid of a gate projection,
+    then projected out.  ``gate_cap`` None leaves the gates' pre-activations uncapped."""
+    dim: int
+    n_heads: int
+    key_dim: int
+    value_dim: int
+    eps: float
+    gate_cap: Optional[float] = None
+    den_eps: float = 1e-6
+    kind: str = "matrix_memory"
+
+
+@dataclass(frozen=True)
 class GatedFeedForwardSpec:
-    """w2( act(w1 x) * (w3 x) ) without biases (reference model.py:219-227)."""
+    """w2( act(w1 x) * (w3 x) ) without biases (reference model.py:219-227); ``activation``
+    "silu" or "gelu_tanh"."""
     dim: int
     hidden: int
     activation: str = "silu"
@@ -70,12 +121,13 @@ class GatedFeedForwardSpec:
 class LayerSpec:
     """One block.  ``arrangement`` names how norms, mixer, feed-forward and the residual
     stream are wired ("pre_norm": reference model.py:161-164).  ``name`` is the prefix of
-    the layer's tensors.  Parameter sub-names are those of the arrangement."""
+    the layer's tensors.  Parameter sub-names are those of the arrangement.  A block whose
+    ``feed_forward`` is None has the mixer's sublayer only."""
     name: str
     mixer: object
     mixer_norm: NormSpec
-    feed_forward: object
-    feed_forward_norm: NormSpec
+    feed_forward: object = None
+    feed_forward_norm: Optional[NormSpec] = None
     arrangement: str = "pre_norm"
     mixer_name: str = "mixer"
     mixer_norm_name: str = "mixer_norm"

@@ -578,9 +578,16 @@ extern "C" int gfa_attention_generic(const void* q, const void* k_pages, const v
 }
 
 // --------------------------------------------------------------------------------------
-// gate: out[n, i] = act(gu[n, i]) * gu[n, I + i], act = silu (model.py:227)
-template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I,
+// gate: out[n, i] = act(gu[n, i]) * gu[n, I + i]; act 0 = silu (model.py:227), 1 = the tanh
+// form of gelu, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+template <int ACT>
+__device__ __forceinline__ float gate_act(float a) {
+    if (ACT == 0) return a / (1.f + expf(-a));
+    return 0.5f * a * (1.f + tanhf(0.7978845608028654f * (a + 0.044715f * a * a * a)));
+}
+
+template <typename T, int ACT>
+__global__ void gate_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I,
                                 size_t total) {
     for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < total;
          e += (size_t)gridDim.x * blockDim.x) {
@@ -588,12 +595,13 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
         const int i = (int)(e % I);
         const float a = load_as_float(gu + n * 2 * I + i);
         const float b = load_as_float(gu + n * 2 * I + I + i);
-        store_from_float(out + e, (a / (1.f + expf(-a))) * b);
+        store_from_float(out + e, gate_act<ACT>(a) * b);
     }
 }
 
 // bfloat16 rows whose width is a multiple of 8: eight elements per thread, 16-byte accesses
-__global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu,
+template <int ACT>
+__global__ __launch_bounds__(256) void gate_mul_bf16x8_kernel(const bf16_t* __restrict__ gu,
                                                               bf16_t* __restrict__ out, int I8,
                                                               size_t total8) {
     const size_t e = blockIdx.x * (size_t)256 + threadIdx.x;
@@ -606,29 +614,40 @@ __global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __re
     uint4 o;
     bf16_t* oe = (bf16_t*)&o;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const float x = bf16_to_float(ae[j]);
-        oe[j] = float_to_bf16((x / (1.f + expf(-x))) * bf16_to_float(be[j]));
-    }
+    for (int j = 0; j < 8; ++j)
+        oe[j] = float_to_bf16(gate_act<ACT>(bf16_to_float(ae[j])) * bf16_to_float(be[j]));
     ((uint4*)out)[e] = o;
 }
 
-extern "C" int gfa_silu_mul(const void* gu, void* out, int n_rows, int I, int is_bf16,
-                            hipStream_t stream) {
+template <int ACT>
+static int launch_gate_mul(const void* gu, void* out, int n_rows, int I, int is_bf16,
+                           hipStream_t stream) {
     const size_t total = (size_t)n_rows * I;
     if (total == 0) return 0;
     if (is_bf16 && I % 8 == 0) {
         const size_t total8 = total / 8;
-        silu_mul_bf16x8_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, stream>>>(
+        gate_mul_bf16x8_kernel<ACT><<<(unsigned)((total8 + 255) / 256), 256, 0, stream>>>(
             (const bf16_t*)gu, (bf16_t*)out, I / 8, total8);
         return GFA_LAUNCH_RESULT();
     }
     const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
     if (is_bf16)
-        silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
+        gate_mul_kernel<bf16_t, ACT><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
     else
-        silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
+        gate_mul_kernel<float, ACT><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
     return GFA_LAUNCH_RESULT();
+}
+
+extern "C" int gfa_gate_mul(const void* gu, void* out, int n_rows, int I, int act, int is_bf16,
+                            hipStream_t stream) {
+    if (act == 0) return launch_gate_mul<0>(gu, out, n_rows, I, is_bf16, stream);
+    if (act == 1) return launch_gate_mul<1>(gu, out, n_rows, I, is_bf16, stream);
+    return (int)hipErrorInvalidValue;
+}
+
+extern "C" int gfa_silu_mul(const void* gu, void* out, int n_rows, int I, int is_bf16,
+                            hipStream_t stream) {
+    return launch_gate_mul<0>(gu, out, n_rows, I, is_bf16, stream);
 }
 
 // --------------------------------------------------------------------------------------

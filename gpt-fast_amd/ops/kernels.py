@@ -229,18 +229,30 @@ def attention_generic(q: torch.Tensor, k_pages, v_pages, tok_seq, tok_pos, table
 
 
 # ----------------------------------------------------------------------------- elementwise
-def silu_mul(gu: torch.Tensor, out: Optional[torch.Tensor] = None):
-    """out[n, i] = silu(gu[n, i]) * gu[n, I + i]; gu [N, 2I]."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def gate_mul(gu: torch.Tensor, activation: str = "silu", out: Optional[torch.Tensor] = None):
+    """out[n, i] = act(gu[n, i]) * gu[n, I + i]; gu [N, 2I]; act "silu" or "gelu_tanh"
+    (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))))."""
     require_device(gu)
     require_contiguous(gu=gu)
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"gate activation '{activation}': {sorted(GATE_ACTIVATIONS)}")
     n, two_i = gu.shape
     if two_i % 2:
-        raise KernelError("silu_mul: the row width must be even")
+        raise KernelError("gate_mul: the row width must be even")
     if out is None:
         out = torch.empty((n, two_i // 2), dtype=gu.dtype, device=gu.device)
-    check(library("core").gfa_silu_mul(ptr(gu), ptr(out), _i(n), _i(two_i // 2),
-                                       _i(_is_bf16(gu)), stream_handle()), "silu_mul")
+    check(library("core").gfa_gate_mul(ptr(gu), ptr(out), _i(n), _i(two_i // 2),
+                                       _i(GATE_ACTIVATIONS[activation]), _i(_is_bf16(gu)),
+                                       stream_handle()), "gate_mul")
     return out
+
+
+def silu_mul(gu: torch.Tensor, out: Optional[torch.Tensor] = None):
+    """out[n, i] = silu(gu[n, i]) * gu[n, I + i]; gu [N, 2I]."""
+    return gate_mul(gu, "silu", out)
 
 
 def add_into(residual: torch.Tensor, y: torch.Tensor):

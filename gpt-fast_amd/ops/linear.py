@@ -253,9 +253,17 @@ def _linear_into(x, w, residual):
     return K.add_into(residual, torch.matmul(x, w.t()))
 
 
-def gated_linear(x: torch.Tensor, w13: torch.Tensor):
-    """[M, I] = silu(x W1^T) * (x W3^T), with w13 = rows of W1 then rows of W3
-    (model.py:227)."""
+GATE_ACTIVATIONS = K.GATE_ACTIVATIONS
+
+
+def gated_linear(x: torch.Tensor, w13: torch.Tensor, activation: str = "silu"):
+    """[M, I] = act(x W1^T) * (x W3^T), with w13 = rows of W1 then rows of W3
+    (model.py:227).  The products whose epilogue applies the gate know silu; another
+    activation runs the product, then the gate kernel."""
+    if activation != "silu":
+        if isinstance(x, HalfNormed):
+            raise KernelError("a norm in two halves feeds the silu gate's kernels only")
+        return K.gate_mul(linear(x, w13), activation)
     if isinstance(x, HalfNormed):
         return _fast().skinny_after_chain_gated(x.xg, x.ssq, x.eps, w13)
     if x.dtype == torch.float32:
@@ -272,15 +280,16 @@ def gated_linear(x: torch.Tensor, w13: torch.Tensor):
 
 
 def gated_into(x, w13: torch.Tensor, w2: torch.Tensor, residual: torch.Tensor, then_norm=None,
-               takes_halves: bool = False):
-    """residual += (silu(x W1^T) * (x W3^T)) W2^T: :func:`gated_linear`, then
+               takes_halves: bool = False, activation: str = "silu"):
+    """residual += (act(x W1^T) * (x W3^T)) W2^T: :func:`gated_linear`, then
     :func:`linear_into` with its arguments and result.  Between two few-row kernels that take
     and leave a norm in halves, the gate's result stays in the order the second one loads it
     in (``gemm_bf16.ChunkedRows``)."""
-    if isinstance(x, HalfNormed) and _chains(x.shape[0], x.dtype, w2, then_norm, takes_halves):
+    if activation == "silu" and isinstance(x, HalfNormed) \
+            and _chains(x.shape[0], x.dtype, w2, then_norm, takes_halves):
         h = _fast().skinny_after_chain_gated(x.xg, x.ssq, x.eps, w13, chunked=True)
     else:
-        h = gated_linear(x, w13)
+        h = gated_linear(x, w13, activation)
     return linear_into(h, w2, residual, then_norm, takes_halves)
 
 

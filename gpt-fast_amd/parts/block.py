@@ -6,20 +6,24 @@ from .base import FEED_FORWARDS, MIXERS, NORMS, Part, ResidualStream, Runtime, r
 class PreNormBlock(Part):
     """``h = x + mixer(norm1(x)); out = h + ffn(norm2(h))`` (reference model.py:161-164).
     The residual stream is float32 and updated in place; the sums happen in the
-    parts' epilogues."""
+    parts' epilogues.  A spec without a feed-forward gives ``out = h``."""
 
     def __init__(self, spec: LayerSpec, runtime: Runtime):
         self.spec = spec
         self.mixer_norm = NORMS.build(spec.mixer_norm, runtime)
         self.mixer = MIXERS.build(spec.mixer, runtime)
-        self.feed_forward_norm = NORMS.build(spec.feed_forward_norm, runtime)
-        self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, runtime)
+        self.feed_forward_norm = self.feed_forward = None
+        if spec.feed_forward is not None:
+            self.feed_forward_norm = NORMS.build(spec.feed_forward_norm, runtime)
+            self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, runtime)
 
     def children(self):
         s = self.spec
-        return {s.mixer_norm_name: self.mixer_norm, s.mixer_name: self.mixer,
-                s.feed_forward_norm_name: self.feed_forward_norm,
-                s.feed_forward_name: self.feed_forward}
+        out = {s.mixer_norm_name: self.mixer_norm, s.mixer_name: self.mixer}
+        if self.feed_forward is not None:
+            out[s.feed_forward_norm_name] = self.feed_forward_norm
+            out[s.feed_forward_name] = self.feed_forward
+        return out
 
     def parameters(self):
         out = {}
@@ -68,8 +72,9 @@ class PreNormBlock(Part):
         stream = residual if isinstance(residual, ResidualStream) else ResidualStream(residual)
         x = stream.normed(self.mixer_norm, reader=self.mixer)
         self.mixer.forward(x, batch, entry, self._residual_for(self.mixer, stream))
-        h = stream.normed(self.feed_forward_norm, reader=self.feed_forward)
-        self.feed_forward.forward(h, batch, self._residual_for(self.feed_forward, stream))
+        if self.feed_forward is not None:
+            h = stream.normed(self.feed_forward_norm, reader=self.feed_forward)
+            self.feed_forward.forward(h, batch, self._residual_for(self.feed_forward, stream))
         if stream is not residual:
             stream.tensor                    # a caller with a plain tensor gets the sums now
 

@@ -5,12 +5,13 @@ from .base import Param, Part, Runtime, add_late, check_bound, register_feed_for
 
 
 class GatedFeedForward(Part):
-    """``w2( silu(w1 x) * (w3 x) )`` without biases.  w1 and w3 are one matrix ``w13``
-    (rows of w1, then rows of w3) so that the gate is applied where the products end."""
+    """``w2( act(w1 x) * (w3 x) )`` without biases, act = silu or the tanh form of gelu.  w1
+    and w3 are one matrix ``w13`` (rows of w1, then rows of w3) so that the gate is applied
+    where the products end."""
 
     def __init__(self, spec: GatedFeedForwardSpec, runtime: Runtime):
-        if spec.activation != "silu":
-            raise ValueError(f"activation '{spec.activation}': only silu has a kernel")
+        if spec.activation not in L.GATE_ACTIVATIONS:
+            raise ValueError(f"activation '{spec.activation}': {sorted(L.GATE_ACTIVATIONS)}")
         self.spec = spec
         self.rt = runtime
         self.w13 = self.w2 = None
@@ -28,7 +29,9 @@ class GatedFeedForward(Part):
     # x may be an ops.linear.HalfNormed, from one row on (the least number of rows; with the
     # weights streamed past the caches the matrix-core kernel that takes the halves is as fast
     # at one row as the dot-product kernel that does not, and the norm kernel is saved)
-    takes_prepared = 1
+    @property
+    def takes_prepared(self):
+        return 1 if self.spec.activation == "silu" else False
 
     def step_flops(self, q_lens, starts) -> float:
         return 2.0 * sum(q_lens) * 3 * self.spec.hidden * self.spec.dim
@@ -37,7 +40,7 @@ class GatedFeedForward(Part):
         # both products wait until the stream is read next: whether the gate's result stays in
         # the order the second product loads it in depends on the norm that follows
         add_late(residual, lambda rows, then_norm, takes_halves: L.gated_into(
-            x, self.w13, self.w2, rows, then_norm, takes_halves))
+            x, self.w13, self.w2, rows, then_norm, takes_halves, self.spec.activation))
 
 
 register_feed_forward("gated", GatedFeedForward)

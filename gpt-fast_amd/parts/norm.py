@@ -7,9 +7,10 @@ from .base import Param, Part, Runtime, check_bound, register_norm
 
 
 class RMSNorm(Part):
-    """``x * rsqrt(mean(x^2) + eps) * weight`` over the last dimension; statistics and
-    scaling in float32 from the float32 residual stream, one rounding to the compute type
-    at the store.  ``eps`` and the width are the spec's."""
+    """``x * rsqrt(mean(x^2) + eps) * (weight + weight_offset)`` over the last dimension;
+    statistics and scaling in float32 from the float32 residual stream, one rounding to the
+    compute type at the store.  ``eps``, the width and the offset (1 for weights stored
+    around zero) are the spec's; the offset is added once, when the weight is bound."""
 
     replayable = True
 
@@ -19,11 +20,15 @@ class RMSNorm(Part):
         self.weight = None
 
     def parameters(self):
-        return {"weight": Param((self.spec.dim,), role="vector", init="norm")}
+        init = "around_zero" if getattr(self.spec, "weight_offset", 0.0) else "norm"
+        return {"weight": Param((self.spec.dim,), role="vector", init=init)}
 
     def bind(self, tensors):
         check_bound("RMSNorm", self.parameters(), tensors)
         self.weight = tensors["weight"].to(torch.float32).contiguous()
+        offset = float(getattr(self.spec, "weight_offset", 0.0))
+        if offset:
+            self.weight = self.weight + offset
 
     def forward(self, residual: torch.Tensor, rows=None) -> torch.Tensor:
         return K.rmsnorm(residual, self.weight, self.spec.eps, self.rt.dtype, rows=rows)

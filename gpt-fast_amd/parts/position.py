@@ -38,7 +38,12 @@ def llama3_scaled(freqs: torch.Tensor, factor: float, low_freq_factor: float,
                        torch.where(wavelen > low_wavelen, freqs / factor, blended))
 
 
-FREQUENCY_SCALINGS = {"llama3": llama3_scaled}
+def linear_scaled(freqs: torch.Tensor, factor: float, **_ignored) -> torch.Tensor:
+    """Position interpolation: every frequency divided by ``factor``."""
+    return freqs / float(factor)
+
+
+FREQUENCY_SCALINGS = {"llama3": llama3_scaled, "linear": linear_scaled}
 
 
 class RotaryPosition(Part):

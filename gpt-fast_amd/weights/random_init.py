@@ -24,6 +24,8 @@ def _tensor_seed(seed: int, name: str) -> int:
 INITS = {
     "linear": lambda t, std, norm_std: t.mul_(std),                    # N(0, std)
     "norm": lambda t, std, norm_std: t.mul_(norm_std).add_(1.0),       # 1 + N(0, norm_std)
+    "around_zero": lambda t, std, norm_std: t.mul_(norm_std),          # N(0, norm_std)
+    "unit": lambda t, std, norm_std: t,                                # N(0, 1)
 }
 
 
