@@ -112,6 +112,15 @@ def _library_partial_sums(x: torch.Tensor, w: torch.Tensor, S: int) -> torch.Ten
     return torch.bmm(xs, ws, out_dtype=torch.float32)
 
 
+def pad_rows(w: torch.Tensor, multiple: int) -> torch.Tensor:
+    """``w`` [N, K] with zero rows added up to the next multiple: a product with it has that
+    many columns, of which the last are zero."""
+    extra = -w.shape[0] % multiple
+    if not extra:
+        return w
+    return torch.cat([w, w.new_zeros((extra, w.shape[1]))]).contiguous()
+
+
 class HalfNormed:
     """Rows of an RMS norm in two halves, as the few-row product that completed the residual
     stream left them: ``xg`` = bfloat16(residual * norm weight) (``gemm_bf16.ChunkedRows``
@@ -169,7 +178,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     M = x.shape[0]
     if M <= SKINNY_MAX_ROWS:
         return _fast().skinny(x, w, out_dtype=out_dtype)
-    t = _tiled_for(M, w)
+    # the kernel that adds a sliced product's partial sums stores four columns at a time
+    t = _tiled_for(M, w) if out_dtype == torch.float32 or w.shape[0] % 4 == 0 else None
     if t is not None:
         from . import gemm_tiled_bf16 as T
         if out_dtype == torch.float32:

@@ -61,7 +61,8 @@ class DifferentialAttention(Part):
 
     def bind(self, tensors):
         check_bound("DifferentialAttention", self.parameters(), tensors)
-        self.w_in, self.wo = tensors["w_in"], tensors["wo"]
+        # zero rows up to a multiple of eight: the products' kernels store whole groups
+        self.w_in, self.wo = L.pad_rows(tensors["w_in"], 8), tensors["wo"]
         v = {n: tensors[n].to(torch.float32) for n in ("lq1", "lk1", "lq2", "lk2")}
         # one number for the layer, float32
         lam = (torch.exp((v["lq1"] * v["lk1"]).sum()) - torch.exp((v["lq2"] * v["lk2"]).sum())

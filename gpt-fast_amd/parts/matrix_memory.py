@@ -1,4 +1,6 @@
 """Recurrent mixer with a matrix memory per head (the mLSTM cell of xLSTM)."""
+import dataclasses
+
 import torch
 
 from ..cache.store import StateNeed
@@ -32,19 +34,22 @@ class MatrixMemory(Part):
             raise ValueError(f"matrix memory: key_dim {spec.key_dim} > {M.MAX_KEY_DIM}")
         self.spec = spec
         self.rt = runtime
-        self.rows = M.RowLayout.fused(spec.n_heads, spec.key_dim, spec.value_dim)
+        rows = M.RowLayout.fused(spec.n_heads, spec.key_dim, spec.value_dim)
+        self.in_rows = rows.width                       # rows of w_in as it is stored
+        self.rows = dataclasses.replace(rows, width=(rows.width + 7) // 8 * 8)
         self.w_in = self.wo = self.norm = self.gate_bias = None
 
     def parameters(self):
         s = self.spec
-        return {"w_in": Param((self.rows.width, s.dim)),
+        return {"w_in": Param((self.in_rows, s.dim)),
                 "gate_bias": Param((2 * s.n_heads,), role="vector", init="unit"),
                 "norm": Param((s.n_heads * s.value_dim,), role="vector", init="norm"),
                 "wo": Param((s.dim, s.n_heads * s.value_dim))}
 
     def bind(self, tensors):
         check_bound("MatrixMemory", self.parameters(), tensors)
-        self.w_in, self.wo = tensors["w_in"], tensors["wo"]
+        # zero rows up to a multiple of eight: the products' kernels store whole groups
+        self.w_in, self.wo = L.pad_rows(tensors["w_in"], 8), tensors["wo"]
         self.norm = tensors["norm"].to(torch.float32).contiguous()
         self.gate_bias = tensors["gate_bias"].to(torch.float32).contiguous()
 
@@ -56,7 +61,7 @@ class MatrixMemory(Part):
         s = self.spec
         n = sum(q_lens)
         cell = 2.0 * 2.0 * s.n_heads * s.key_dim * s.value_dim          # update and read of S
-        return n * (2.0 * (self.rows.width + s.n_heads * s.value_dim) * s.dim + cell)
+        return n * (2.0 * (self.in_rows + s.n_heads * s.value_dim) * s.dim + cell)
 
     def forward(self, x, batch, entry, residual):
         s = self.spec

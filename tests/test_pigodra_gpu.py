@@ -1,0 +1,433 @@
+"""Pigodra on the GPU against the plain float64 implementation of tests/plain_pigodra.py:
+each mechanism's kernels alone, whole prompts, prompts in portions, token-by-token decoding,
+unequal batches, slots and pages that come back, windows' and kept keys' edges with weights
+that make one key stand out, long memory, and greedy generation through the library's
+generation loop and command line."""
+import math
+
+import pytest
+import torch
+
+import plain_pigodra as P
+import util
+from pigodra_cases import CASES, make_folder
+from util import TOL_BF16, TOL_F32, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+# The memory cell sums a sequence in another order than the plain token-by-token loop does in
+# float64; a float32 engine stays within this of it over a few hundred tokens.
+TOL_F32_LONG = 1e-4
+
+
+def row_errors(got, want):
+    """Per row: root mean square of the difference over that of all of ``want``."""
+    got, want = got.double().cpu(), want.double().cpu()
+    return (got - want).pow(2).mean(-1).sqrt() / want.pow(2).mean().sqrt()
+
+
+def bf16_close(got, want):
+    """A bfloat16 engine against float64 (or against itself, cut or batched another way, where
+    other kernels round at other places).  Rows differ in how much they amplify a rounding
+    error (a head's result is divided by its own size, which may be small), so the bulk of the
+    rows is held to the tolerance and every row to a bound that a wrong key, a lost state or
+    a missing term would still break."""
+    e = row_errors(got, want)
+    return float(e.quantile(0.9)) < TOL_BF16 and float(e.max()) < 0.35
+
+
+def close(got, want, dtype, tol):
+    return bf16_close(got, want) if dtype == "bfloat16" else rel_err(got, want) < tol
+
+
+def _engine(folder, dtype, **kw):
+    import gpt_fast_amd as gfa
+    kw.setdefault("max_tokens", 4096)
+    return gfa.Engine.from_folder(folder, dtype=dtype, device=DEV, **kw)
+
+
+def _steps(eng, toks, cuts, want_all=True):
+    """Feed ``toks`` as one sequence in portions that end at ``cuts``; logits of every token."""
+    import gpt_fast_amd as gfa
+    slot = eng.start_sequence()
+    out, lo = [], 0
+    for hi in list(cuts) + [len(toks)]:
+        if hi <= lo:
+            continue
+        out.append(eng.step([gfa.Entry(slot, toks[lo:hi], want=list(range(hi - lo)))]).cpu())
+        lo = hi
+    eng.end_sequence(slot)
+    return torch.cat(out)
+
+
+# --------------------------------------------------------------------------- mechanisms alone
+def test_gelu_gate_kernel():
+    from gpt_fast_amd.ops import kernels as K
+    torch.manual_seed(0)
+    for dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 1e-2)):
+        for width in (24, 37 * 2):
+            gu = (torch.randn(19, width, device=DEV) * 3).to(dtype)
+            got = K.gate_mul(gu, "gelu_tanh").double().cpu()
+            g = gu.double().cpu()
+            want = P.gelu_tanh(g[:, :width // 2]) * g[:, width // 2:]
+            assert rel_err(got, want) < tol
+            assert rel_err(K.gate_mul(gu, "silu").double().cpu(),
+                           torch.nn.functional.silu(g[:, :width // 2]) * g[:, width // 2:]) < tol
+
+
+def test_norm_with_weights_stored_around_zero():
+    from gpt_fast_amd.config.spec import NormSpec
+    from gpt_fast_amd.parts.base import NORMS, Runtime
+    torch.manual_seed(1)
+    norm = NORMS.build(NormSpec(50, 1e-3, weight_offset=1.0), Runtime(torch.float32, DEV))
+    w = torch.randn(50, device=DEV) * 0.3
+    norm.bind({"weight": w})
+    x = torch.randn(7, 50, device=DEV) * 4
+    want = P.rms_norm_around_zero(x.double().cpu(), w.double().cpu(), 1e-3)
+    assert rel_err(norm.forward(x), want) < 1e-6
+    rows = torch.tensor([5, 0], dtype=torch.int32, device=DEV)
+    assert rel_err(norm.forward(x, rows=rows), want[[5, 0]]) < 1e-6
+
+
+@pytest.mark.parametrize("H,dk,dv,cap", [(2, 16, 32, 8.0), (1, 24, 40, None), (3, 20, 12, 3.0),
+                                         (2, 72, 8, 15.0), (1, 130, 33, 5.0)])
+def test_memory_cell_kernels_alone(H, dk, dv, cap):
+    """Three sequences of unequal length in one launch, then a second launch that goes on
+    from the state the first one left, in other slots than their order."""
+    from gpt_fast_amd.ops import matrix_memory as M
+    torch.manual_seed(H * 100 + dk)
+    rows = M.RowLayout.fused(H, dk, dv)
+    lens1, lens2 = [5, 1, 37], [1, 9, 2]
+    slots = [4, 0, 2]
+    state = torch.zeros(6, M.state_size(H, dk, dv), device=DEV)
+    state[1].fill_(7.0)                                        # a slot nobody uses stays as it is
+    bias = torch.randn(2 * H, device=DEV)
+    weight = 1 + 0.2 * torch.randn(H * dv, device=DEV)
+    seqs = [torch.randn(a + b, rows.width, device=DEV) * 1.5 for a, b in zip(lens1, lens2)]
+    for s in seqs:
+        s[:, rows.i:] *= 3                                    # gates that move
+    got = [[] for _ in seqs]
+    for part, lens in ((0, lens1), (1, lens2)):
+        chunks = [s[:l] if part == 0 else s[-l:] for s, l in zip(seqs, lens)]
+        proj = torch.cat(chunks).contiguous()
+        q_start = torch.tensor([sum(lens[:b]) for b in range(len(lens) + 1)], dtype=torch.int32, device=DEV)
+        o = M.scan(proj, rows, bias, state, q_start, torch.tensor(slots, dtype=torch.int32, device=DEV),
+                   3, H, dk, dv, dk ** -0.5, cap or 0.0, 1e-6)
+        y = M.head_norm_gate(o, weight, proj, rows, 1e-5, torch.float32)
+        at = 0
+        for b, l in enumerate(lens):
+            got[b].append(y[at:at + l].double().cpu())
+            at += l
+    assert torch.all(state[1] == 7.0)
+    for b, s in enumerate(seqs):
+        p = s.double().cpu()
+        T = p.shape[0]
+        q = p[:, rows.q:rows.k].view(T, H, dk) * dk ** -0.5
+        k = p[:, rows.k:rows.v].view(T, H, dk)
+        v = p[:, rows.v:rows.g].view(T, H, dv)
+        bi, bf = bias[:H].double().cpu(), bias[H:].double().cpu()
+        capped = (lambda z: z) if cap is None else (lambda z: cap * torch.tanh(z / cap))
+        ig = capped(p[:, rows.i:rows.f] + bi)
+        fg = torch.nn.functional.logsigmoid(capped(p[:, rows.f:] + bf))
+        o, (S, n, m) = P.matrix_memory_cell(q, k, v, ig, fg)
+        want = (P.unit_rms(o, 1e-5).reshape(T, H * dv) * weight.double().cpu()
+                * torch.sigmoid(p[:, rows.g:rows.i]))
+        assert rel_err(torch.cat(got[b]), want) < 2e-5
+        st = state[slots[b]].double().cpu()
+        assert rel_err(st[:H * dk * dv].view(H, dk, dv), S) < 2e-5
+        assert rel_err(st[H * dk * dv:H * dk * (dv + 1)].view(H, dk), n) < 2e-5
+        assert rel_err(st[H * dk * (dv + 1):], m) < 2e-5
+
+
+def _attention_alone(dtype, H, G, dim, vdim, window, first, rot, lens, starts, boost=None):
+    """The rotation, cache write and attention kernels over sequences that already hold
+    ``starts[b]`` tokens and get ``lens[b]`` more, against the plain attention.  ``boost``:
+    (sequence, key position, factor) multiplies that key's rows, so that its score stands out."""
+    from gpt_fast_amd.ops import differential_attention as DA
+    from gpt_fast_amd.parts.position import rotary_frequencies
+    torch.manual_seed(dim * 7 + vdim)
+    width = H * 2 * dim + G * 2 * dim + G * vdim + H
+    k_off, v_off, g_off = H * 2 * dim, H * 2 * dim + G * 2 * dim, H * 2 * dim + G * 2 * dim + G * vdim
+    total = [s + l for s, l in zip(starts, lens)]
+    n_pages = sum((t + 63) // 64 for t in total)
+    k_pages = torch.zeros(n_pages, G, 64, 2 * dim, device=DEV, dtype=dtype)
+    v_pages = torch.zeros(n_pages, G, vdim, 64, device=DEV, dtype=dtype)
+    # pages handed out in an order that is not the sequences' own
+    order = list(range(n_pages))[::-1]
+    tables, at = [], 0
+    for t in total:
+        n = (t + 63) // 64
+        tables.append(order[at:at + n])
+        at += n
+    widest = max(len(t) for t in tables)
+    table = torch.tensor([t + [-1] * (widest - len(t)) for t in tables], dtype=torch.int32, device=DEV)
+    freqs = (rotary_frequencies(rot, 777.0) / 1.5).to(DEV) if rot else None
+    seqs = [(torch.randn(t, width, device=DEV) * 1.2).to(dtype) for t in total]
+    if boost is not None:
+        b, key, factor = boost
+        seqs[b][key, k_off:v_off] *= factor
+    lam, eps, scale, out_scale = 0.37, 1e-5, 0.4, 0.7
+    got = []
+    for phase in (0, 1):                         # what was there before, then the new tokens
+        rows, seq_of, pos_of = [], [], []
+        for b, s in enumerate(seqs):
+            lo, hi = (0, starts[b]) if phase == 0 else (starts[b], total[b])
+            rows.append(s[lo:hi])
+            seq_of += [b] * (hi - lo)
+            pos_of += list(range(lo, hi))
+        if not seq_of:
+            continue
+        proj = torch.cat(rows).contiguous()
+        tok_seq = torch.tensor(seq_of, dtype=torch.int32, device=DEV)
+        tok_pos = torch.tensor(pos_of, dtype=torch.int32, device=DEV)
+        q = DA.rope_store(proj, 0, k_off, v_off, freqs, tok_seq, tok_pos, table, k_pages, v_pages,
+                          H, G, dim, vdim, rot)
+        if phase == 1:
+            y = DA.attention_generic(q, k_pages, v_pages, proj[:, g_off:g_off + H], tok_seq, tok_pos,
+                                     table, scale, window, first, lam, eps, out_scale)
+            at = 0
+            for b in range(len(seqs)):
+                got.append(y[at:at + lens[b]].double().cpu())
+                at += lens[b]
+    worst = 0.0
+    for b, s in enumerate(seqs):
+        p = s.double().cpu()
+        T = p.shape[0]
+        m = {"heads": H, "kv_heads": G, "dim": dim, "vdim": vdim, "diff": 1 - out_scale, "scale": scale,
+             "mask": {"size": window or None, "keep_first": first},
+             "rot": {"dims": rot, "base": 777.0, "scaling": {"factor": 1.5}}}
+        # the plain attention from projections: identity weights pick q, k, v, g out of the rows
+        w = {"q": torch.eye(width, dtype=P.F)[:k_off], "k": torch.eye(width, dtype=P.F)[k_off:v_off],
+             "v": torch.eye(width, dtype=P.F)[v_off:g_off], "g": torch.eye(width, dtype=P.F)[g_off:],
+             "o": torch.eye(H * vdim, dtype=P.F)}
+        # lambda = exp(a) - exp(0) + diff = 0.37
+        a = math.log(lam - (1 - out_scale) + 1.0)
+        w.update(lq1=torch.tensor([a], dtype=P.F), lk1=torch.tensor([1.0], dtype=P.F),
+                 lq2=torch.zeros(1, dtype=P.F), lk2=torch.zeros(1, dtype=P.F))
+        want = P.differential_attention(p, w, "", m, eps)[starts[b]:]
+        worst = max(worst, rel_err(got[b], want))
+    return worst
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+@pytest.mark.parametrize("H,G,dim,vdim,window,first,rot", [
+    (4, 2, 16, 32, 24, 3, 16), (3, 1, 24, 24, 7, 0, 8), (2, 2, 20, 40, 90, 70, 20),
+    (6, 3, 8, 16, 0, 0, 0), (2, 1, 32, 64, 64, 1, 16), (1, 1, 36, 18, 65, 64, 12)])
+def test_attention_kernels_alone(dtype, tol, H, G, dim, vdim, window, first, rot):
+    # prompts from the start, portions at an offset, single tokens far into a sequence
+    assert _attention_alone(dtype, H, G, dim, vdim, window, first, rot, [150, 1, 70], [0, 0, 0]) < tol
+    assert _attention_alone(dtype, H, G, dim, vdim, window, first, rot, [1, 33, 1, 2], [199, 100, 0, 63]) < tol
+
+
+@pytest.mark.parametrize("offset", [0, -1])
+@pytest.mark.parametrize("decode", [False, True])
+def test_a_loud_key_at_the_windows_edge_and_among_the_kept_keys(offset, decode):
+    """One key's rows are multiplied by 30: where it is visible it takes nearly all the weight
+    of a map.  The last token (position 139) has a window of 40: key 100 is the last one inside,
+    key 99 is outside; with 5 kept keys, key 4 is kept and key 5 is not.  The same with the
+    last token fed alone after the others, and with the key on a page's border."""
+    H, G, dim, vdim, window, first = 2, 1, 16, 16, 40, 5
+    lens, starts = ([1], [139]) if decode else ([140], [0])
+    for key in (100 + offset, 4 - offset * 1):
+        err = _attention_alone(torch.float32, H, G, dim, vdim, window, first, 8, lens, starts,
+                               boost=(0, key, 30.0))
+        assert err < 5e-5
+    # a window whose first key is the first key of a page, a sequence of exactly two pages
+    lens, starts = ([1], [127]) if decode else ([128], [0])
+    for key in (64 + offset, 63, 0):
+        assert _attention_alone(torch.float32, H, G, dim, vdim, 64, 1, 8, lens, starts,
+                                boost=(0, key, 30.0)) < 5e-5
+    # the test can see a mask that is one key off: the plain results differ by far more
+    torch.manual_seed(0)
+    m = {"heads": 1, "kv_heads": 1, "dim": 4, "vdim": 4, "diff": 0.3, "scale": 1.0,
+         "mask": {"size": 40, "keep_first": 5}, "rot": {"dims": 0}}
+    w = {n: torch.randn(s, 6, dtype=P.F) for n, s in (("q", 8), ("k", 8), ("v", 4), ("g", 1))}
+    w.update(o=torch.eye(4, dtype=P.F), lq1=torch.zeros(1, dtype=P.F), lk1=torch.zeros(1, dtype=P.F),
+             lq2=torch.zeros(1, dtype=P.F), lk2=torch.zeros(1, dtype=P.F))
+    h = torch.randn(140, 6, dtype=P.F)
+    h[99] *= 30
+    a = P.differential_attention(h, w, "", m, 1e-6)[139]
+    m["mask"]["size"] = 41
+    assert rel_err(P.differential_attention(h, w, "", m, 1e-6)[139], a) > 1e-2
+
+
+# --------------------------------------------------------------------------- whole models
+@pytest.mark.parametrize("name", ["A", "B", "M", "T"])
+@pytest.mark.parametrize("dtype,tol", [("float32", TOL_F32_LONG), ("bfloat16", TOL_BF16)])
+def test_whole_prompt_matches_plain_at_every_position(tmp_path, name, dtype, tol):
+    folder = make_folder(tmp_path, name, seed=11)
+    cfg, w = P.load_folder(folder)
+    toks = util.random_tokens(cfg["vocab"], 230, 3)
+    outs = []
+    want = P.forward(w, cfg, toks, outs)
+    eng = _engine(folder, dtype)
+    got = _steps(eng, toks, [])
+    assert close(got, want, dtype, tol)
+    if dtype == "float32":
+        # one token, and the first tokens of a sequence
+        assert rel_err(_steps(eng, toks[:1], []), want[:1]) < TOL_F32
+        assert rel_err(_steps(eng, toks[:3], []), want[:3]) < TOL_F32
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("dtype,tol,same", [("float32", TOL_F32_LONG, 2e-5), ("bfloat16", TOL_BF16, TOL_BF16)])
+def test_portions_and_token_by_token_equal_the_whole_prompt(tmp_path, name, dtype, tol, same):
+    folder = make_folder(tmp_path, name, seed=12)
+    cfg, w = P.load_folder(folder)
+    toks = util.random_tokens(cfg["vocab"], 210, 5)
+    want = P.forward(w, cfg, toks)
+    eng = _engine(folder, dtype)
+    whole = _steps(eng, toks, [])
+    assert close(whole, want, dtype, tol)
+    for cuts in ([2, 4, 5, 70, 128, 129], [63, 64, 65, 192], [17, 150], list(range(150, 210)),
+                 list(range(1, 80))):
+        got = _steps(eng, toks, cuts)
+        assert close(got, want, dtype, tol), cuts
+        assert close(got, whole, dtype, same), cuts
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("dtype,same", [("float32", 1e-5), ("bfloat16", TOL_BF16)])
+def test_unequal_batches_equal_each_request_alone(tmp_path, name, dtype, same):
+    import gpt_fast_amd as gfa
+    folder = make_folder(tmp_path, name, seed=13)
+    cfg, w = P.load_folder(folder)
+    lens = [1, 5, 131, 64, 70]
+    tail = 30
+    seqs = [util.random_tokens(cfg["vocab"], n + tail, 40 + n) for n in lens]
+    eng = _engine(folder, dtype, max_tokens=64 * 20, max_sequences=6)
+    alone = [_steps(eng, s, [n] + list(range(n + 1, n + tail))) for s, n in zip(seqs, lens)]
+    slots = [eng.start_sequence() for _ in seqs]
+    got = [[] for _ in seqs]
+    out = eng.step([gfa.Entry(sl, s[:n], want=list(range(n))) for sl, s, n in zip(slots, seqs, lens)]).cpu()
+    at = 0
+    for b, n in enumerate(lens):
+        got[b].append(out[at:at + n])
+        at += n
+    live = list(range(len(seqs)))
+    for t in range(tail):
+        if t == 10:                                  # a shorter request ends earlier
+            eng.end_sequence(slots[1])
+            live.remove(1)
+        out = eng.step([gfa.Entry(slots[b], [seqs[b][lens[b] + t]], want=[0]) for b in live]).cpu()
+        for i, b in enumerate(live):
+            got[b].append(out[i:i + 1])
+    for b in live:
+        eng.end_sequence(slots[b])
+    eng.cache.check()
+    for b, s in enumerate(seqs):
+        g = torch.cat(got[b])
+        assert close(g, alone[b][:g.shape[0]], dtype, same), b
+    want = P.forward(w, cfg, seqs[2])
+    assert close(torch.cat(got[2]), want, dtype, TOL_F32_LONG)
+
+
+def test_slots_and_pages_that_come_back_start_clean(tmp_path):
+    """A cache of few pages and two slots: requests follow one another in the same slots and
+    pages, long decoding gives the window's pages back, and every request equals the plain
+    computation of itself alone."""
+    import gpt_fast_amd as gfa
+    folder = make_folder(tmp_path, "A", seed=14)
+    cfg, w = P.load_folder(folder)
+    eng = _engine(folder, "float32", max_tokens=64 * 7, max_sequences=2)
+    for round_ in range(3):
+        a = util.random_tokens(cfg["vocab"], 150 + 90, 60 + round_)
+        b = util.random_tokens(cfg["vocab"], 40 + 90, 70 + round_)
+        sa, sb = eng.start_sequence(), eng.start_sequence()
+        assert {sa, sb} == {0, 1}
+        got_a, got_b = [], []
+        out = eng.step([gfa.Entry(sa, a[:150], want=[149]), gfa.Entry(sb, b[:40], want=[39])]).cpu()
+        got_a.append(out[0:1])
+        got_b.append(out[1:2])
+        for t in range(89):
+            out = eng.step([gfa.Entry(sa, [a[150 + t]], want=[0]), gfa.Entry(sb, [b[40 + t]], want=[0])]).cpu()
+            got_a.append(out[0:1])
+            got_b.append(out[1:2])
+        eng.cache.check()
+        eng.end_sequence(sb)
+        eng.end_sequence(sa)
+        assert rel_err(torch.cat(got_a), P.forward(w, cfg, a[:-1])[149:]) < TOL_F32_LONG
+        assert rel_err(torch.cat(got_b), P.forward(w, cfg, b[:-1])[39:]) < TOL_F32_LONG
+    for _, g in eng.cache.kv_groups:
+        assert g.pages.held == 0
+
+
+def test_a_memory_written_far_back_is_read_hundreds_of_tokens_later(tmp_path):
+    """Forget gates close to one and an input gate that opens for few tokens: what the
+    state holds after 500 tokens comes from the first of them.  Decoding the last 40 alone
+    reads it through the carried state; a state that was lost or reset would show."""
+    def patch(t):
+        for name in t:
+            if name.endswith("mix.f.b"):
+                t[name] = torch.full_like(t[name], 9.0)
+            if name.endswith("mix.i.b"):
+                t[name] = torch.full_like(t[name], -4.0)
+            if name.endswith("mix.i"):
+                t[name] = t[name] * 12
+    folder = make_folder(tmp_path, "M", seed=15, patch=patch, tag="far")
+    cfg, w = P.load_folder(folder)
+    toks = util.random_tokens(cfg["vocab"], 540, 9)
+    want = P.forward(w, cfg, toks)
+    # it matters: the same tokens without the first 300 give other logits at the end
+    assert rel_err(P.forward(w, cfg, toks[300:])[-40:], want[-40:]) > 1e-2
+    for dtype, tol in (("float32", TOL_F32_LONG), ("bfloat16", TOL_BF16)):
+        eng = _engine(folder, dtype)
+        got = _steps(eng, toks, [500] + list(range(501, 540)))
+        assert close(got[-41:], want[-41:], dtype, tol)
+        assert close(got, want, dtype, tol)
+
+
+def test_peaked_softmax_over_a_long_prompt_and_decoding_past_the_window(tmp_path):
+    """Scores scaled up until a map's weight sits on one or two keys, among some hundred
+    candidates or at the window's edge; then 130 tokens decoded one by one, so that the
+    window (100 and 24) passes over decoded tokens and pages are given back."""
+    def patch(t):
+        for name in t:
+            if name.endswith("mix.q") and t[name].shape[0] > 100:
+                t[name] = t[name] * 6
+    folder = make_folder(tmp_path, "A", seed=16, patch=patch, tag="peaked")
+    cfg, w = P.load_folder(folder)
+    toks = util.random_tokens(cfg["vocab"], 400, 21)
+    want = P.forward(w, cfg, toks)
+    for dtype in ("float32", "bfloat16"):
+        eng = _engine(folder, dtype, max_tokens=64 * 8, max_sequences=1)
+        got = _steps(eng, toks, [270] + list(range(271, 400)))
+        if dtype == "float32":
+            assert rel_err(got, want) < TOL_F32_LONG
+        else:
+            # scores six times as large carry six times the rounding of q and k into the
+            # softmax: bfloat16 is held to the typical row only
+            assert float(row_errors(got, want).median()) < TOL_BF16
+        eng.cache.check()
+
+
+# --------------------------------------------------------------------------- generation
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_loop_and_the_recorded_step(tmp_path, name):
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.engine.generate import generate
+    folder = make_folder(tmp_path, name, seed=17)
+    cfg, w = P.load_folder(folder)
+    prompts = [util.random_tokens(cfg["vocab"], n, 80 + n) for n in (7, 1, 90, 30)]
+    want = [P.greedy_generate(w, cfg, p, 12) for p in prompts]
+    eng = _engine(folder, "float32", max_tokens=64 * 12, max_sequences=4)
+    for use_graph in (False, True, True):                       # the recording is replayed
+        got = generate(eng, prompts, max_new_tokens=12, temperature=0.0, use_graph=use_graph)
+        assert got.tokens == want, use_graph
+    # two at a time: slots and state come back between the batches
+    got = generate(eng, prompts, max_new_tokens=12, temperature=0.0, batch_size=2)
+    assert got.tokens == want
+    eng.cache.check()
+
+
+def test_command_line_entry_point(tmp_path):
+    import gpt_fast_amd as gfa
+    folder = make_folder(tmp_path, "B", seed=18)
+    cfg, w = P.load_folder(folder)
+    prompt = util.random_tokens(cfg["vocab"], 20, 1)
+    lines = []
+    res = gfa.main(prompt=prompt, num_samples=1, max_new_tokens=8, temperature=0.0, top_k=None,
+                   checkpoint_path=folder, dtype="float32", device=DEV, out=lines.append)
+    assert res["result"].tokens[0] == P.greedy_generate(w, cfg, prompt, 8)
+    assert any("tokens/sec" in str(l) for l in lines)
