@@ -10,7 +10,9 @@ JSON line: ``value`` is decoded tokens per second; ``prefill`` is one 2,048-toke
 the live sequences) per second with the HBM peak; ``points`` holds decode at batch 1 and 64;
 ``vs_baseline`` compares the batch-1 point with the reference's published batch-1 number.
 
-Other workloads of the same program: ``--preset`` (another shape), ``--context`` (cache
+Other workloads of the same program: ``--preset`` (another shape, also of another
+architecture: ``pigodra-4096`` is a Pigodra stack with the width, inner size and head sizes of
+``llama-3.1-8b``; with ``--layers N`` both run their first N layers), ``--context`` (cache
 positions per sequence), ``--prompt-lens LO:HI`` (prompts of unequal, seeded random lengths;
 adds the ragged prefill's tokens per second), ``--prefill-only`` (just the timed prompt, for
 profiling), ``--parts`` (no model: a layer's products at ``--batch`` rows and the prompt
@@ -93,9 +95,10 @@ def decode_run(engine, prompt_lens, warmup, steps, use_graph=True, warm_prefill=
     dt = per_run[median_run]
     sess.close()
     # bytes of the median run's middle step: weights once + keys and values of every live token
-    ctx = sum(n + warmup + median_run * steps + steps // 2 for n in prompt_lens)
-    kv_bytes = sum(g.bytes_per_token() for _, g in engine.cache.kv_groups) * ctx
-    step_bytes = engine.model.parameter_bytes() + kv_bytes
+    # (a window bounds the keys a step reads; a fixed-size state is read and written whole)
+    lengths = [n + warmup + median_run * steps + steps // 2 for n in prompt_lens]
+    cache_bytes = sum(g.step_bytes(n) for g in engine.cache.groups for n in lengths)
+    step_bytes = engine.model.parameter_bytes() + cache_bytes
     for s in slots:
         engine.end_sequence(s)
     return dt, step_bytes, prefill_seconds, per_run
@@ -247,12 +250,14 @@ def main():
 
     arch, cfg = gfa.find_preset(args.preset, args.architecture)
     raw = arch.config_dict(cfg)
-    full_layers = raw[arch.layer_count_key]
+    # the layers are a number, or a list with one entry per layer
+    listed = isinstance(raw[arch.layer_count_key], list)
+    full_layers = len(raw[arch.layer_count_key]) if listed else raw[arch.layer_count_key]
     if args.layers:
-        raw[arch.layer_count_key] = args.layers
+        raw[arch.layer_count_key] = raw[arch.layer_count_key][:args.layers] if listed else args.layers
         cfg = arch.read_config(raw)
     sizes = dict(arch.describe(cfg)) if arch.describe is not None else {}
-    n_layers = raw[arch.layer_count_key]
+    n_layers = len(raw[arch.layer_count_key]) if listed else raw[arch.layer_count_key]
     batch, context = args.batch, args.context
     if args.parts:
         print(json.dumps({"metric": f"kernels alone; {args.preset} bf16", "rows": batch,
@@ -275,6 +280,8 @@ def main():
     log(f"[bench] model ready in {time.time() - t0:.1f} s")
 
     model_name = "Llama-3.1-8B" if args.preset == "llama-3.1-8b" else args.preset
+    if args.layers:
+        model_name += f" ({n_layers} of {full_layers} layers)"
     # the reference's published number is for this shape only
     headline = args.preset == "llama-3.1-8b" and not args.layers
     use_graph = not args.no_graph

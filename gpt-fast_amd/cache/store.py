@@ -94,6 +94,11 @@ class Group:
         """Bytes a one-token step reads of this group per cached token."""
         return 0
 
+    def step_bytes(self, length: int) -> int:
+        """Bytes a one-token step reads and writes of this group for one sequence that holds
+        ``length`` tokens."""
+        return self.bytes_per_token() * length
+
     def snapshot(self) -> Optional[Callable[[], None]]:
         """What puts the group's contents back after a step is run twice (the warm-up of a
         recording); None if a repeated step writes the same bytes."""
@@ -126,6 +131,11 @@ class KVGroup(Group):
     def bytes_per_token(self) -> int:
         return (self.entries * self.need.n_kv_heads * (self.need.head_dim + self.need.v_dim)
                 * self.k.element_size())
+
+    def step_bytes(self, length: int) -> int:
+        if self.need.window is not None:
+            length = min(length, self.need.window + self.need.keep_first)
+        return self.bytes_per_token() * length
 
     def acquire(self, slot):
         self.held[slot] = []
@@ -202,6 +212,9 @@ class StateGroup(Group):
         # that only fill a fixed shape read and write it
         self.data = torch.zeros((entries, geometry.n_slots + 1) + tuple(need.shape),
                                 dtype=getattr(torch, need.dtype), device=device)
+
+    def step_bytes(self, length: int) -> int:
+        return 2 * self.data[:, 0].numel() * self.data.element_size()
 
     def acquire(self, slot):
         self.data[:, slot].zero_()

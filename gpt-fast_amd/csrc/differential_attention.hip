@@ -209,3 +209,279 @@ extern "C" int gfa_da_attention_generic(const void* q, const void* k_pages, cons
             scale, window, keep_first, lam, eps, out_scale);
     return GFA_LAUNCH_RESULT();
 }
+
+// --------------------------------------------------------------------------------------
+// The same on the matrix cores, bfloat16, for head sizes in eights up to 128 and value sizes
+// in sixteens up to 256 (the cache orders of common.h that those sizes have).
+//
+// A wavefront owns 16 rows of one sequence and kv head; a row is a (token, query head of the
+// kv head's group) pair, heads fastest.  It walks the visible keys in blocks of 32 - the
+// blocks of the kept first keys, then those of the window - with a running maximum and sum
+// per row and map, all float.  Both products are formed transposed, so that every operand is
+// read in the order the cache has and the weights never leave their registers:
+//   S^T = K Q^T   A = 16 keys x 32 dims of a key page, B = Q^T from registers;
+//   O^T = V^T P^T A = 16 dims x 32 keys of a value page, B = the eight weights a lane holds.
+// v_mfma_f32_16x16x32_bf16: lane l supplies row (A) / column (B) l % 16, k = 8 (l / 16) .. +7,
+// and receives rows 4 (l / 16) .. +3 of column l % 16; with the key order of common.h those
+// rows of the two 16-key tiles are the lane's keys 8 (l / 16) .. +7 of the block.
+// Head sizes that are no multiple of 32 and value sizes below the template's are filled up:
+// the query's registers are zero there and the loads are pointed at valid elements.
+//
+// SPLIT (one token per sequence, a group of at most 16 heads): the waves of a workgroup share
+// the blocks of one tile of rows and the first wave adds their partial results in wave order.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 da_bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float da_floatx4_t;
+union DAFrag {
+    uint4 u;
+    bf16_t e[8];
+    da_bf16x8_t v;
+};
+
+__device__ __forceinline__ float da_max_lane_groups(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16, GFA_WAVE));
+    return fmaxf(v, __shfl_xor(v, 32, GFA_WAVE));
+}
+__device__ __forceinline__ float da_sum_lane_groups(float v) {
+    v += __shfl_xor(v, 16, GFA_WAVE);
+    return v + __shfl_xor(v, 32, GFA_WAVE);
+}
+
+template <int DK, int DVT, bool SPLIT>
+__global__ __launch_bounds__(SPLIT ? 512 : 256) void da_attention_mfma_kernel(
+        const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+        const bf16_t* __restrict__ v_pages, const bf16_t* __restrict__ gate, int gate_stride,
+        const int* __restrict__ q_start, const int* __restrict__ start_pos,
+        const int* __restrict__ table, int table_stride, bf16_t* __restrict__ out, int H, int G,
+        int dim, int vdim, float scale_log2, int window, int keep_first, float lam, float eps,
+        float out_scale) {
+    extern __shared__ float da_lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nw = blockDim.x >> 6;
+    const int li = lane & 15, lg = lane >> 4;
+    const int g = blockIdx.y, seq = blockIdx.z;
+    const int Rg = H / G;
+    const int q0 = q_start[seq];
+    const int rows_total = (q_start[seq + 1] - q0) * Rg;
+    const int row0 = SPLIT ? 0 : (blockIdx.x * nw + wave) * 16;
+    if (!SPLIT && row0 >= rows_total) return;          // no barrier follows without SPLIT
+    const int spos = start_pos[seq];
+    const int* pages = table + (size_t)seq * table_stride;
+    const bool row_ok = row0 + li < rows_total;
+    const int row = row_ok ? row0 + li : rows_total - 1;
+    const int tok = row / Rg, head = g * Rg + row % Rg;
+    const int pos = spos + tok;
+    const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+
+    DAFrag qf[DA_MAPS][DK];
+    const bf16_t* qrow = q + ((size_t)(q0 + tok) * H + head) * DA_MAPS * dim;
+#pragma unroll
+    for (int a = 0; a < DA_MAPS; ++a)
+#pragma unroll
+        for (int kk = 0; kk < DK; ++kk) {
+            const int d = kk * 32 + lg * 8;
+            qf[a][kk].u = d < dim ? *(const uint4*)(qrow + a * dim + d) : make_uint4(0, 0, 0, 0);
+        }
+
+    // blocks of 32 keys that some row of this wave sees
+    const int last_row = row0 + 15 < rows_total ? row0 + 15 : rows_total - 1;
+    const int p_min = spos + row0 / Rg, p_max = spos + last_row / Rg;
+    const int win_lo = (window > 0 && p_min - window + 1 > 0) ? p_min - window + 1 : 0;
+    const int n_first = keep_first < win_lo ? keep_first : win_lo;
+    const int a_end = (n_first + 31) / 32;
+    const int b_begin = win_lo / 32 > a_end ? win_lo / 32 : a_end;
+    const int n_blocks = a_end + (p_max / 32 + 1 - b_begin);
+    const int vtiles = vdim / 16;
+
+    da_floatx4_t o[DA_MAPS][DVT];
+    float m[DA_MAPS], l[DA_MAPS];
+#pragma unroll
+    for (int a = 0; a < DA_MAPS; ++a) {
+        m[a] = -INFINITY;
+        l[a] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DVT; ++dt) o[a][dt] = da_floatx4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    for (int it = SPLIT ? wave : 0; it < n_blocks; it += SPLIT ? nw : 1) {
+        const int bi = it < a_end ? it : b_begin + (it - a_end);
+        const int page = pages[bi >> 1];
+        const bf16_t* kb = k_pages + cache_region(page, g, G, DA_MAPS * dim) + (size_t)(bi & 1) * 32 * dim;
+        const bf16_t* vb = v_pages + cache_region(page, g, G, vdim) + (size_t)(bi & 1) * 512;
+        // slots beyond the newest key this wave reads may hold no data yet: their weight is
+        // zero, and so must their value be (whatever bits lie there)
+        uint4 keep;
+        {
+            const int key0 = bi * 32 + lg * 8;
+            auto two = [&](int e) {
+                return (key0 + e <= p_max ? 0xffffu : 0u) | (key0 + e + 1 <= p_max ? 0xffff0000u : 0u);
+            };
+            keep = make_uint4(two(0), two(2), two(4), two(6));
+        }
+        DAFrag pf[DA_MAPS];
+        float alpha[DA_MAPS];
+#pragma unroll
+        for (int a = 0; a < DA_MAPS; ++a) {
+            da_floatx4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < DK; ++kk) {
+                const int chunk = kk * 4 + lg;
+                const int c = chunk * 8 < dim ? chunk : 0;
+                const bf16_t* src = kb + (size_t)a * GFA_PAGE * dim + c * 256 + li * 8;
+                DAFrag k0, k1;
+                k0.u = *(const uint4*)src;
+                k1.u = *(const uint4*)(src + 128);
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.v, qf[a][kk].v, s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.v, qf[a][kk].v, s1, 0, 0, 0);
+            }
+            float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+            float mx = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int j = bi * 32 + lg * 8 + e;
+                const bool see = j <= pos && (j >= lo || j < keep_first);
+                sv[e] = see ? sv[e] * scale_log2 : -INFINITY;
+                mx = fmaxf(mx, sv[e]);
+            }
+            mx = da_max_lane_groups(mx);
+            const float m_new = fmaxf(m[a], mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            alpha[a] = exp2f(m[a] - m_use);
+            float ps = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p = exp2f(sv[e] - m_use);
+                ps += p;
+                pf[a].e[e] = float_to_bf16(p);
+            }
+            l[a] = l[a] * alpha[a] + ps;
+            m[a] = m_new;
+        }
+#pragma unroll
+        for (int dt = 0; dt < DVT; ++dt) {
+            const int dtc = dt < vtiles ? dt : vtiles - 1;
+            DAFrag vf;
+            vf.u = *(const uint4*)(vb + (size_t)dtc * 1024 + lg * 128 + li * 8);
+            vf.u.x &= keep.x;
+            vf.u.y &= keep.y;
+            vf.u.z &= keep.z;
+            vf.u.w &= keep.w;
+#pragma unroll
+            for (int a = 0; a < DA_MAPS; ++a) {
+                o[a][dt] *= alpha[a];
+                o[a][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[a].v, o[a][dt], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < DA_MAPS; ++a) l[a] = da_sum_lane_groups(l[a]);
+
+    if (SPLIT) {
+        // per wave: m and l of 16 rows and two maps, then O [map][dim][row < rows_total]
+        const int per_wave = 64 + DA_MAPS * vdim * rows_total;
+        float* mine = da_lds + (size_t)wave * per_wave;
+        if (lg == 0) {
+#pragma unroll
+            for (int a = 0; a < DA_MAPS; ++a) {
+                mine[a * 32 + li] = m[a];
+                mine[a * 32 + 16 + li] = l[a];
+            }
+        }
+        if (row_ok) {
+#pragma unroll
+            for (int a = 0; a < DA_MAPS; ++a)
+#pragma unroll
+                for (int dt = 0; dt < DVT; ++dt)
+                    if (dt < vtiles)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            mine[64 + ((size_t)a * vdim + dt * 16 + lg * 4 + j) * rows_total + li] = o[a][dt][j];
+        }
+        __syncthreads();
+        if (wave != 0) return;
+#pragma unroll
+        for (int a = 0; a < DA_MAPS; ++a) {
+            float M = -INFINITY;
+            for (int w = 0; w < nw; ++w) M = fmaxf(M, da_lds[(size_t)w * per_wave + a * 32 + li]);
+            float L = 0.f;
+#pragma unroll
+            for (int dt = 0; dt < DVT; ++dt) o[a][dt] = da_floatx4_t{0.f, 0.f, 0.f, 0.f};
+            for (int w = 0; w < nw; ++w) {
+                const float* theirs = da_lds + (size_t)w * per_wave;
+                const float mw = theirs[a * 32 + li];
+                const float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
+                L += theirs[a * 32 + 16 + li] * f;
+                if (row_ok) {
+#pragma unroll
+                    for (int dt = 0; dt < DVT; ++dt)
+                        if (dt < vtiles)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j)
+                                o[a][dt][j] += f * theirs[64 + ((size_t)a * vdim + dt * 16 + lg * 4 + j) * rows_total + li];
+                }
+            }
+            l[a] = L;
+        }
+    }
+
+    // a1 - lam a2, the head's norm, the gate
+    const float inv0 = 1.f / l[0], inv1 = lam / l[1];
+    float ss = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt)
+        if (dt < vtiles)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float v = o[0][dt][j] * inv0 - o[1][dt][j] * inv1;
+                o[0][dt][j] = v;
+                ss = fmaf(v, v, ss);
+            }
+    ss = da_sum_lane_groups(ss);
+    float f = rsqrtf(ss / (float)vdim + eps) * out_scale;
+    if (gate) f *= 1.f / (1.f + expf(-bf16_to_float(gate[(size_t)(q0 + tok) * gate_stride + head])));
+    if (!row_ok) return;
+    bf16_t* orow = out + ((size_t)(q0 + tok) * H + head) * vdim;
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt)
+        if (dt < vtiles) {
+            union { uint2 u; bf16_t e[4]; } w;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w.e[j] = float_to_bf16(o[0][dt][j] * f);
+            *(uint2*)(orow + dt * 16 + lg * 4) = w.u;
+        }
+}
+
+// rows_max: the most rows (tokens times heads of a group) any sequence of the step brings.
+// split_waves > 0: one token per sequence, that many waves share a tile's blocks.
+extern "C" int gfa_da_attention_mfma(const void* q, const void* k_pages, const void* v_pages,
+                                     const void* gate, int gate_stride, const int* q_start,
+                                     const int* start_pos, const int* table, int table_stride,
+                                     void* out, int n_seqs, int rows_max, int H, int G, int dim,
+                                     int vdim, float scale, int window, int keep_first, float lam,
+                                     float eps, float out_scale, int split_waves,
+                                     hipStream_t stream) {
+    if (n_seqs <= 0 || rows_max <= 0) return 0;
+    if (dim % 8 || dim > 128 || vdim % 16 || vdim > 256 || n_seqs > 65535 || G > 65535 || H % G)
+        return (int)hipErrorInvalidValue;
+    const int Rg = H / G;
+    if (split_waves > 0 && (Rg > 16 || rows_max != Rg || split_waves > 8)) return (int)hipErrorInvalidValue;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    const int dk = dim <= 32 ? 1 : dim <= 64 ? 2 : 4, dvt = vdim <= 64 ? 4 : vdim <= 128 ? 8 : 16;
+    const dim3 grid(split_waves > 0 ? 1 : (rows_max + 63) / 64, G, n_seqs);
+    const int threads = split_waves > 0 ? split_waves * 64 : 256;
+    const size_t shmem = split_waves > 0 ? (size_t)split_waves * (64 + DA_MAPS * vdim * Rg) * sizeof(float) : 0;
+    if (shmem > 64 * 1024) return (int)hipErrorInvalidValue;
+#define DA_LAUNCH(K_, V_, S_) da_attention_mfma_kernel<K_, V_, S_><<<grid, threads, shmem, stream>>>( \
+        (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (const bf16_t*)gate, \
+        gate_stride, q_start, start_pos, table, table_stride, (bf16_t*)out, H, G, dim, vdim, \
+        scale_log2, window, keep_first, lam, eps, out_scale)
+#define DA_PICK_V(K_, S_) do { if (dvt == 4) DA_LAUNCH(K_, 4, S_); else if (dvt == 8) DA_LAUNCH(K_, 8, S_); \
+        else DA_LAUNCH(K_, 16, S_); } while (0)
+#define DA_PICK(S_) do { if (dk == 1) DA_PICK_V(1, S_); else if (dk == 2) DA_PICK_V(2, S_); \
+        else DA_PICK_V(4, S_); } while (0)
+    if (split_waves > 0) DA_PICK(true);
+    else DA_PICK(false);
+#undef DA_PICK
+#undef DA_PICK_V
+#undef DA_LAUNCH
+    return GFA_LAUNCH_RESULT();
+}

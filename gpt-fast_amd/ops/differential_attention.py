@@ -95,8 +95,76 @@ def attention_generic(q, k_pages, v_pages, gate, tok_seq, tok_pos, table, scale,
     return out
 
 
+MFMA_MAX_DIM, MFMA_MAX_VDIM = 128, 256
+SPLIT_MAX_WAVES = 8
+LDS_BYTES = 64 * 1024
+
+
+def mfma_takes(q, k_pages, v_pages) -> bool:
+    """The matrix-core kernel's shapes: bfloat16, head sizes in eights up to 128, value sizes
+    in sixteens up to 256."""
+    dim, vdim = q.shape[3], v_pages.shape[2]
+    return (q.dtype == torch.bfloat16 and dim % 8 == 0 and dim <= MFMA_MAX_DIM
+            and vdim % 16 == 0 and vdim <= MFMA_MAX_VDIM)
+
+
+def split_waves_for(heads_per_group: int, vdim: int) -> int:
+    """Waves that share one sequence's keys in a step of one token per sequence: as many as
+    their partial results fit the workgroup's shared memory, at most eight; 0: not available."""
+    if heads_per_group > 16:
+        return 0
+    per_wave = (64 + MAPS * vdim * heads_per_group) * 4
+    return min(SPLIT_MAX_WAVES, LDS_BYTES // per_wave)
+
+
+def attention_mfma(q, k_pages, v_pages, gate, q_start, start_pos, table, n_seqs, max_q_len,
+                   scale, window, keep_first, lam, eps, out_scale, single_tokens=False):
+    """As :func:`attention_generic`, on the matrix cores; sequences are given by ``q_start``
+    [n_seqs + 1] (first row of each) and ``start_pos`` [n_seqs] (tokens cached before the
+    step).  ``single_tokens``: every sequence brings one token, and the waves of a workgroup
+    share its keys."""
+    require_device(q, k_pages, v_pages, gate, q_start, start_pos, table)
+    require_contiguous(q=q, q_start=q_start, start_pos=start_pos, table=table)
+    n, H, maps, dim = q.shape
+    G, vdim = k_pages.shape[1], v_pages.shape[2]
+    if maps != MAPS or H % G or not mfma_takes(q, k_pages, v_pages):
+        raise KernelError(f"differential attention on the matrix cores: q {tuple(q.shape)}, "
+                          f"values of {vdim}, {G} kv heads")
+    _check_pages(k_pages, v_pages, G, dim, vdim, q.dtype)
+    for name, t in (("q_start", q_start), ("start_pos", start_pos), ("table", table)):
+        if t.dtype != torch.int32:
+            raise KernelError(f"{name} must be int32")
+    if q_start.numel() < n_seqs + 1 or start_pos.numel() < n_seqs or table.shape[0] < n_seqs:
+        raise KernelError("differential attention: the step's description is shorter than the batch")
+    gate_stride = 0
+    if gate is not None:
+        if gate.shape != (n, H) or gate.dtype != q.dtype or (H > 1 and gate.stride(1) != 1):
+            raise KernelError("differential attention: gate must be [N, H] of q's type")
+        gate_stride = gate.stride(0)
+    waves = 0
+    if single_tokens:
+        waves = split_waves_for(H // G, vdim)
+        if n != n_seqs or max_q_len != 1 or waves < 1:
+            raise KernelError("differential attention: single_tokens needs one row per sequence")
+    out = torch.empty((n, H * vdim), dtype=q.dtype, device=q.device)
+    check(library("differential_attention").gfa_da_attention_mfma(
+        ptr(q), ptr(k_pages), ptr(v_pages), ptr(gate), _i(gate_stride), ptr(q_start), ptr(start_pos),
+        ptr(table), _i(table.shape[1]), ptr(out), _i(n_seqs), _i(max_q_len * (H // G)), _i(H), _i(G),
+        _i(dim), _i(vdim), _f(scale), _i(window or 0), _i(keep_first), _f(lam), _f(eps),
+        _f(out_scale), _i(waves), stream_handle()), "da_attention_mfma")
+    return out
+
+
 def attention(q, k_pages, v_pages, gate, batch, table, scale, window, keep_first, lam, eps,
               out_scale):
-    """Which kernel runs a step's differential attention: the plain one, for every shape."""
+    """Which kernel runs a step's differential attention.  float32 engine, and shapes the
+    matrix-core kernel refuses: the plain kernel.  bfloat16: the matrix-core kernel, with the
+    waves of a workgroup sharing a sequence's keys when every sequence brings one token."""
+    if mfma_takes(q, k_pages, v_pages):
+        H, G, vdim = q.shape[1], k_pages.shape[1], v_pages.shape[2]
+        single = bool(batch.is_decode) and split_waves_for(H // G, vdim) >= 1
+        return attention_mfma(q, k_pages, v_pages, gate, batch.q_start, batch.start_pos, table,
+                              batch.n_seqs, batch.max_q_len, scale, window, keep_first, lam, eps,
+                              out_scale, single_tokens=single)
     return attention_generic(q, k_pages, v_pages, gate, batch.tok_seq, batch.tok_pos, table,
                              scale, window, keep_first, lam, eps, out_scale)

@@ -139,7 +139,8 @@ def test_memory_cell_kernels_alone(H, dk, dv, cap):
         assert rel_err(st[H * dk * (dv + 1):], m) < 2e-5
 
 
-def _attention_alone(dtype, H, G, dim, vdim, window, first, rot, lens, starts, boost=None):
+def _attention_alone(dtype, H, G, dim, vdim, window, first, rot, lens, starts, boost=None,
+                     kernel="plain"):
     """The rotation, cache write and attention kernels over sequences that already hold
     ``starts[b]`` tokens and get ``lens[b]`` more, against the plain attention.  ``boost``:
     (sequence, key position, factor) multiplies that key's rows, so that its score stands out."""
@@ -182,9 +183,18 @@ def _attention_alone(dtype, H, G, dim, vdim, window, first, rot, lens, starts, b
         tok_pos = torch.tensor(pos_of, dtype=torch.int32, device=DEV)
         q = DA.rope_store(proj, 0, k_off, v_off, freqs, tok_seq, tok_pos, table, k_pages, v_pages,
                           H, G, dim, vdim, rot)
-        if phase == 1:
+        if phase == 1 and kernel == "plain":
             y = DA.attention_generic(q, k_pages, v_pages, proj[:, g_off:g_off + H], tok_seq, tok_pos,
                                      table, scale, window, first, lam, eps, out_scale)
+        elif phase == 1:
+            # the matrix-core kernel; with one token per sequence also its form in which the
+            # waves of a workgroup share the keys
+            q_start = torch.tensor([sum(lens[:b]) for b in range(len(lens) + 1)], dtype=torch.int32, device=DEV)
+            start_pos = torch.tensor(starts, dtype=torch.int32, device=DEV)
+            y = DA.attention_mfma(q, k_pages, v_pages, proj[:, g_off:g_off + H], q_start, start_pos,
+                                  table, len(lens), max(lens), scale, window, first, lam, eps, out_scale,
+                                  single_tokens=kernel == "shared")
+        if phase == 1:
             at = 0
             for b in range(len(seqs)):
                 got.append(y[at:at + lens[b]].double().cpu())
@@ -217,6 +227,37 @@ def test_attention_kernels_alone(dtype, tol, H, G, dim, vdim, window, first, rot
     # prompts from the start, portions at an offset, single tokens far into a sequence
     assert _attention_alone(dtype, H, G, dim, vdim, window, first, rot, [150, 1, 70], [0, 0, 0]) < tol
     assert _attention_alone(dtype, H, G, dim, vdim, window, first, rot, [1, 33, 1, 2], [199, 100, 0, 63]) < tol
+
+
+@pytest.mark.parametrize("H,G,dim,vdim,window,first,rot", [
+    (4, 2, 16, 32, 24, 3, 16), (6, 3, 8, 16, 0, 0, 0), (2, 1, 32, 64, 64, 1, 16), (4, 1, 48, 48, 33, 2, 8),
+    (2, 2, 128, 256, 70, 65, 64), (8, 2, 64, 128, 0, 0, 32), (3, 3, 96, 80, 100, 4, 96), (16, 1, 24, 16, 5, 1, 0)])
+def test_attention_on_the_matrix_cores_alone(H, G, dim, vdim, window, first, rot):
+    def run(lens, starts, kernel):
+        return _attention_alone(torch.bfloat16, H, G, dim, vdim, window, first, rot, lens, starts, kernel=kernel)
+    assert run([150, 1, 70], [0, 0, 0], "mfma") < 3e-2
+    assert run([1, 33, 1, 2], [199, 100, 0, 63], "mfma") < 3e-2
+    assert run([1, 1, 1, 1, 1], [199, 31, 0, 63, 64], "mfma") < 3e-2
+    assert run([1, 1, 1, 1, 1], [199, 31, 0, 63, 64], "shared") < 3e-2
+    assert run([1], [700], "shared") < 3e-2
+
+
+@pytest.mark.parametrize("offset", [0, -1])
+@pytest.mark.parametrize("decode", [False, True])
+def test_a_loud_key_on_the_matrix_cores(offset, decode):
+    """As below, for the bfloat16 kernels.  Scores thirty times as large carry thirty times
+    the rounding of q and k into the weights, hence the wider bound; a key wrongly seen or
+    missed changes the result by its whole size."""
+    H, G, dim, vdim, window, first = 2, 1, 16, 16, 40, 5
+    lens, starts = ([1], [139]) if decode else ([140], [0])
+    for kernel in ("mfma", "shared") if decode else ("mfma",):
+        for key in (100 + offset, 4 - offset):
+            assert _attention_alone(torch.bfloat16, H, G, dim, vdim, window, first, 8, lens, starts,
+                                    boost=(0, key, 30.0), kernel=kernel) < 0.1
+        lens2, starts2 = ([1], [127]) if decode else ([128], [0])
+        for key in (64 + offset, 63, 0):
+            assert _attention_alone(torch.bfloat16, H, G, dim, vdim, 64, 1, 8, lens2, starts2,
+                                    boost=(0, key, 30.0), kernel=kernel) < 0.1
 
 
 @pytest.mark.parametrize("offset", [0, -1])
