@@ -147,6 +147,232 @@ extern "C" int gfa_matrix_memory_scan(const float* proj, const float* gate_bias,
 }
 
 // --------------------------------------------------------------------------------------
+// The same cell for runs of many tokens, a chunk of MC_L tokens at a time instead of token by
+// token.  Inside a chunk that starts from (S0, n0, m0), with F_t the running sum of the log
+// forget gates from the chunk's start, g_s = i_s - F_s and M_t = max(m0, max_{s<=t} g_s):
+//     m_t = F_t + M_t
+//     S_t^T q_t = exp(m0 - M_t) S0^T q_t + sum_{s<=t} exp(g_s - M_t) (k_s . q_t) v_s
+//     n_t . q_t = exp(m0 - M_t) n0 . q_t + sum_{s<=t} exp(g_s - M_t) (k_s . q_t)
+// and the state after the chunk's last token L is
+//     S_L = exp(m0 - M_L) S0 + sum_s exp(g_s - M_L) k_s v_s^T        (n_L likewise)
+// which is the recurrence written out; every exponent is <= 0.  All float.
+// grid (dv / MC_COLS, H, sequences), 256 threads; q, k, v of the chunk, the weighted scores
+// and the workgroup's columns of S are in shared memory.
+#define MC_L 32
+#define MC_COLS 32
+#define MC_PS (MC_L + 1)
+
+__host__ __device__ inline int mc_row_stride(int dk) {
+    const int dk4 = (dk + 3) / 4 * 4;
+    return (dk4 / 4) % 2 == 0 ? dk4 + 4 : dk4;      // in floats; a quarter of it is odd
+}
+
+__global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
+        const float* __restrict__ proj, const float* __restrict__ gate_bias,
+        float* __restrict__ state, size_t slot_stride, const int* __restrict__ q_start,
+        const int* __restrict__ slots, float* __restrict__ out, MMShape s) {
+    extern __shared__ __attribute__((aligned(16))) float mc_lds[];
+    const int KS = mc_row_stride(s.dk);
+    const int dk4 = (s.dk + 3) / 4 * 4;
+    float* Qs = mc_lds;                          // [MC_L][KS]
+    float* Ks = Qs + MC_L * KS;                  // [MC_L][KS]
+    float* Vs = Ks + MC_L * KS;                  // [MC_L][MC_COLS]
+    float* Ps = Vs + MC_L * MC_COLS;             // [MC_L][MC_PS]
+    float* Ss = Ps + MC_L * MC_PS;               // [dk4][MC_COLS]
+    float* ns = Ss + dk4 * MC_COLS;              // [dk4]
+    float* gs = ns + dk4;                        // [MC_L] g_s
+    float* Ms = gs + MC_L;                       // [MC_L] M_t
+    float* mt = Ms + MC_L;                       // [MC_L] m_t
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col0 = blockIdx.x * MC_COLS;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int t0 = q_start[b], t1 = q_start[b + 1];
+    float* const base = state + (size_t)slots[b] * slot_stride;
+    float* const S = base + (size_t)h * s.dk * s.dv;
+    float* const nvec = base + (size_t)s.H * s.dk * s.dv + (size_t)h * s.dk;
+    float* const mptr = base + (size_t)s.H * s.dk * (s.dv + 1) + h;
+    const float ib = gate_bias[h], fb = gate_bias[s.H + h];
+
+    for (int e = tid; e < dk4 * MC_COLS; e += 256) {
+        const int d = e / MC_COLS, c = e % MC_COLS;
+        Ss[e] = (d < s.dk && col0 + c < s.dv) ? S[(size_t)d * s.dv + col0 + c] : 0.f;
+    }
+    for (int d = tid; d < dk4; d += 256) ns[d] = d < s.dk ? nvec[d] : 0.f;
+    float m_prev = *mptr;
+
+    for (int c0 = t0; c0 < t1; c0 += MC_L) {
+        const int Lc = t1 - c0 < MC_L ? t1 - c0 : MC_L;
+        __syncthreads();                         // the chunk before is done with Qs .. Ss
+        // q (scaled), k, v of the chunk; rows beyond its end and columns beyond dk are zero
+        for (int e = tid; e < MC_L * KS; e += 256) {
+            const int t = e / KS, d = e - t * KS;
+            const bool ok = t < Lc && d < s.dk;
+            const float* row = proj + (size_t)(c0 + t) * s.row_width;
+            Qs[e] = ok ? row[s.q_off + h * s.dk + d] * s.q_scale : 0.f;
+            Ks[e] = ok ? row[s.k_off + h * s.dk + d] : 0.f;
+        }
+        for (int e = tid; e < MC_L * MC_COLS; e += 256) {
+            const int t = e / MC_COLS, c = e % MC_COLS;
+            Vs[e] = (t < Lc && col0 + c < s.dv)
+                ? proj[(size_t)(c0 + t) * s.row_width + s.v_off + h * s.dv + col0 + c] : 0.f;
+        }
+        if (wave == 0) {
+            // the gates of the chunk: running sum of f, running maximum of g, one token per lane
+            const int t = lane;
+            float ig = -INFINITY, fg = 0.f;
+            if (t < Lc) {
+                const float* row = proj + (size_t)(c0 + t) * s.row_width;
+                ig = mm_cap(row[s.i_off + h] + ib, s.cap);
+                fg = mm_logsigmoid(mm_cap(row[s.f_off + h] + fb, s.cap));
+            }
+            float F = fg;
+#pragma unroll
+            for (int o = 1; o < MC_L; o <<= 1) {
+                const float up = __shfl_up(F, o, GFA_WAVE);
+                if (lane >= o) F += up;
+            }
+            const float g = ig - F;
+            float M = fmaxf(g, m_prev);
+#pragma unroll
+            for (int o = 1; o < MC_L; o <<= 1) {
+                const float up = __shfl_up(M, o, GFA_WAVE);
+                if (lane >= o) M = fmaxf(M, up);
+            }
+            if (t < MC_L) {
+                gs[t] = g;
+                Ms[t] = M;
+                mt[t] = F + M;
+            }
+        }
+        __syncthreads();
+        // scores of the chunk, weighted: P[t][s] = (q_t . k_s) exp(g_s - M_t) for s <= t
+        {
+            const int ty = tid >> 4, tx = tid & 15;
+            float a00 = 0.f, a01 = 0.f, a10 = 0.f, a11 = 0.f;
+            const float4* q0 = (const float4*)(Qs + ty * KS);
+            const float4* q1 = (const float4*)(Qs + (ty + 16) * KS);
+            const float4* k0 = (const float4*)(Ks + tx * KS);
+            const float4* k1 = (const float4*)(Ks + (tx + 16) * KS);
+            for (int d = 0; d < dk4 / 4; ++d) {
+                const float4 x0 = q0[d], x1 = q1[d], y0 = k0[d], y1 = k1[d];
+                a00 = fmaf(x0.x, y0.x, fmaf(x0.y, y0.y, fmaf(x0.z, y0.z, fmaf(x0.w, y0.w, a00))));
+                a01 = fmaf(x0.x, y1.x, fmaf(x0.y, y1.y, fmaf(x0.z, y1.z, fmaf(x0.w, y1.w, a01))));
+                a10 = fmaf(x1.x, y0.x, fmaf(x1.y, y0.y, fmaf(x1.z, y0.z, fmaf(x1.w, y0.w, a10))));
+                a11 = fmaf(x1.x, y1.x, fmaf(x1.y, y1.y, fmaf(x1.z, y1.z, fmaf(x1.w, y1.w, a11))));
+            }
+            auto weight = [&](int t, int ss, float a) {
+                return ss <= t ? a * expf(gs[ss] - Ms[t]) : 0.f;    // g of a missing token is -inf
+            };
+            Ps[ty * MC_PS + tx] = weight(ty, tx, a00);
+            Ps[ty * MC_PS + tx + 16] = weight(ty, tx + 16, a01);
+            Ps[(ty + 16) * MC_PS + tx] = weight(ty + 16, tx, a10);
+            Ps[(ty + 16) * MC_PS + tx + 16] = weight(ty + 16, tx + 16, a11);
+        }
+        __syncthreads();
+        // o_t for the workgroup's columns: four columns per thread, eight threads per token
+        {
+            const int t = tid >> 3, j = tid & 7, c4 = j * 4;
+            const float carry = expf(m_prev - Ms[t]);
+            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+            const float* qr = Qs + t * KS;
+            for (int d = 0; d < s.dk; ++d) {
+                const float x = qr[d];
+                const float4 sv = *(const float4*)(Ss + d * MC_COLS + c4);
+                acc.x = fmaf(x, sv.x, acc.x);
+                acc.y = fmaf(x, sv.y, acc.y);
+                acc.z = fmaf(x, sv.z, acc.z);
+                acc.w = fmaf(x, sv.w, acc.w);
+            }
+            acc.x *= carry; acc.y *= carry; acc.z *= carry; acc.w *= carry;
+            const float* pr = Ps + t * MC_PS;
+            for (int ss = 0; ss <= t; ++ss) {
+                const float x = pr[ss];
+                const float4 vv = *(const float4*)(Vs + ss * MC_COLS + c4);
+                acc.x = fmaf(x, vv.x, acc.x);
+                acc.y = fmaf(x, vv.y, acc.y);
+                acc.z = fmaf(x, vv.z, acc.z);
+                acc.w = fmaf(x, vv.w, acc.w);
+            }
+            float nq0 = 0.f, nq1 = 0.f;
+            for (int d = j; d < s.dk; d += 8) nq0 = fmaf(qr[d], ns[d], nq0);
+            for (int ss = j; ss <= t; ss += 8) nq1 += pr[ss];
+            float nq = carry * nq0 + nq1;
+            nq += __shfl_xor(nq, 1, GFA_WAVE);
+            nq += __shfl_xor(nq, 2, GFA_WAVE);
+            nq += __shfl_xor(nq, 4, GFA_WAVE);
+            if (t < Lc) {
+                const float inv = 1.f / (fmaxf(fabsf(nq), expf(-mt[t])) + s.den_eps);
+                float* dst = out + (size_t)(c0 + t) * s.H * s.dv + (size_t)h * s.dv + col0 + c4;
+                const float r[4] = {acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv};
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (col0 + c4 + i < s.dv) dst[i] = r[i];
+            }
+        }
+        __syncthreads();
+        // the state after the chunk's last token
+        {
+            const float M_end = Ms[Lc - 1];
+            const float decay = expf(m_prev - M_end);
+            const int dr = tid >> 3, c4 = (tid & 7) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int d = dr + 32 * i;
+                if (d < s.dk) {
+                    float4 acc = *(const float4*)(Ss + d * MC_COLS + c4);
+                    acc.x *= decay; acc.y *= decay; acc.z *= decay; acc.w *= decay;
+                    for (int ss = 0; ss < Lc; ++ss) {
+                        const float x = expf(gs[ss] - M_end) * Ks[ss * KS + d];
+                        const float4 vv = *(const float4*)(Vs + ss * MC_COLS + c4);
+                        acc.x = fmaf(x, vv.x, acc.x);
+                        acc.y = fmaf(x, vv.y, acc.y);
+                        acc.z = fmaf(x, vv.z, acc.z);
+                        acc.w = fmaf(x, vv.w, acc.w);
+                    }
+                    *(float4*)(Ss + d * MC_COLS + c4) = acc;
+                }
+            }
+            for (int d = tid; d < s.dk; d += 256) {
+                float a = decay * ns[d];
+                for (int ss = 0; ss < Lc; ++ss) a = fmaf(expf(gs[ss] - M_end), Ks[ss * KS + d], a);
+                ns[d] = a;
+            }
+            m_prev = mt[Lc - 1];
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < s.dk * MC_COLS; e += 256) {
+        const int d = e / MC_COLS, c = e % MC_COLS;
+        if (col0 + c < s.dv) S[(size_t)d * s.dv + col0 + c] = Ss[e];
+    }
+    if (blockIdx.x == 0) {
+        for (int d = tid; d < s.dk; d += 256) nvec[d] = ns[d];
+        if (tid == 0) *mptr = m_prev;
+    }
+}
+
+extern "C" int gfa_matrix_memory_chunk_lds(int dk) {
+    const int dk4 = (dk + 3) / 4 * 4;
+    return (int)sizeof(float) * (2 * MC_L * mc_row_stride(dk) + MC_L * MC_COLS + MC_L * MC_PS
+                                 + dk4 * MC_COLS + dk4 + 3 * MC_L);
+}
+
+extern "C" int gfa_matrix_memory_chunks(const float* proj, const float* gate_bias, float* state,
+                                        size_t slot_stride, const int* q_start, const int* slots,
+                                        float* out, int n_seqs, int H, int dk, int dv, int row_width,
+                                        int q_off, int k_off, int v_off, int i_off, int f_off,
+                                        float q_scale, float cap, float den_eps, hipStream_t stream) {
+    if (n_seqs <= 0) return 0;
+    const int shmem = gfa_matrix_memory_chunk_lds(dk);
+    if (dk > 128 || shmem > 64 * 1024 || H > 65535 || n_seqs > 65535) return (int)hipErrorInvalidValue;
+    MMShape s{H, dk, dv, row_width, q_off, k_off, v_off, i_off, f_off, q_scale, cap, den_eps};
+    dim3 grid((dv + MC_COLS - 1) / MC_COLS, H, n_seqs);
+    matrix_memory_chunk_kernel<<<grid, 256, shmem, stream>>>(proj, gate_bias, state, slot_stride,
+                                                             q_start, slots, out, s);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
 // What follows the cell: each head's o is divided by its root mean square (eps inside the
 // root), times a weight per element, times sigmoid of the gate projection; rounded once, to
 // the type of the output projection's operand.  One wave per (token, head).

@@ -41,11 +41,26 @@ def state_size(n_heads: int, key_dim: int, value_dim: int) -> int:
     return n_heads * (key_dim * value_dim + key_dim + 1)
 
 
+CHUNK_MAX_KEY_DIM = 128      # the chunked kernel keeps a chunk's q and k in shared memory
+CHUNKS_FROM_TOKENS = 16      # runs shorter than this go token by token
+
+
+def cell(proj, layout, gate_bias, state, q_start, slots, n_seqs, max_q_len, n_heads, key_dim,
+         value_dim, q_scale, gate_cap, den_eps) -> torch.Tensor:
+    """Which kernel runs the cell: token by token for short runs (single-token steps), a
+    chunk of tokens at a time where some sequence brings many."""
+    chunked = max_q_len >= CHUNKS_FROM_TOKENS and key_dim <= CHUNK_MAX_KEY_DIM
+    return scan(proj, layout, gate_bias, state, q_start, slots, n_seqs, n_heads, key_dim,
+                value_dim, q_scale, gate_cap, den_eps, chunked=chunked)
+
+
 def scan(proj: torch.Tensor, layout: RowLayout, gate_bias: torch.Tensor, state: torch.Tensor,
          q_start: torch.Tensor, slots: torch.Tensor, n_seqs: int, n_heads: int, key_dim: int,
-         value_dim: int, q_scale: float, gate_cap: float, den_eps: float) -> torch.Tensor:
+         value_dim: int, q_scale: float, gate_cap: float, den_eps: float,
+         chunked: bool = False) -> torch.Tensor:
     """The cell over every sequence's new tokens in order; ``state`` [slots, state_size] is
-    read and left updated.  proj float32 [N, layout.width]; returns o float32 [N, H, dv]."""
+    read and left updated.  proj float32 [N, layout.width]; returns o float32 [N, H, dv].
+    ``chunked``: the kernel that takes 32 tokens at a time (key_dim up to 128)."""
     require_device(proj, gate_bias, state, q_start, slots)
     require_contiguous(proj=proj, gate_bias=gate_bias, state=state, q_start=q_start, slots=slots)
     for name, t in (("proj", proj), ("gate_bias", gate_bias), ("state", state)):
@@ -69,7 +84,11 @@ def scan(proj: torch.Tensor, layout: RowLayout, gate_bias: torch.Tensor, state: 
     if key_dim > MAX_KEY_DIM:
         raise KernelError(f"matrix memory: key_dim {key_dim} > {MAX_KEY_DIM} is not supported")
     out = torch.empty((proj.shape[0], n_heads, value_dim), dtype=torch.float32, device=proj.device)
-    check(library("matrix_memory").gfa_matrix_memory_scan(
+    if chunked and key_dim > CHUNK_MAX_KEY_DIM:
+        raise KernelError(f"matrix memory: the chunked kernel takes key_dim up to {CHUNK_MAX_KEY_DIM}")
+    entry = (library("matrix_memory").gfa_matrix_memory_chunks if chunked
+             else library("matrix_memory").gfa_matrix_memory_scan)
+    check(entry(
         ptr(proj), ptr(gate_bias), ptr(state), _sz(state.stride(0)), ptr(q_start), ptr(slots),
         ptr(out), _i(n_seqs), _i(n_heads), _i(key_dim), _i(value_dim), _i(layout.width),
         _i(layout.q), _i(layout.k), _i(layout.v), _i(layout.i), _i(layout.f), _f(q_scale),

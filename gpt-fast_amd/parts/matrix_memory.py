@@ -66,9 +66,9 @@ class MatrixMemory(Part):
     def forward(self, x, batch, entry, residual):
         s = self.spec
         proj = L.linear(x, self.w_in, out_dtype=torch.float32)
-        o = M.scan(proj, self.rows, self.gate_bias, entry.state, batch.q_start, batch.slots,
-                   batch.n_seqs, s.n_heads, s.key_dim, s.value_dim, s.key_dim ** -0.5,
-                   s.gate_cap or 0.0, s.den_eps)
+        o = M.cell(proj, self.rows, self.gate_bias, entry.state, batch.q_start, batch.slots,
+                   batch.n_seqs, batch.max_q_len, s.n_heads, s.key_dim, s.value_dim,
+                   s.key_dim ** -0.5, s.gate_cap or 0.0, s.den_eps)
         y = M.head_norm_gate(o, self.norm, proj, self.rows, s.eps, self.rt.dtype)
         add_late(residual, lambda rows, then_norm, takes_halves: L.linear_into(
             y, self.wo, rows, then_norm, takes_halves))

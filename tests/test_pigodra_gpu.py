@@ -91,13 +91,17 @@ def test_norm_with_weights_stored_around_zero():
 
 @pytest.mark.parametrize("H,dk,dv,cap", [(2, 16, 32, 8.0), (1, 24, 40, None), (3, 20, 12, 3.0),
                                          (2, 72, 8, 15.0), (1, 130, 33, 5.0)])
-def test_memory_cell_kernels_alone(H, dk, dv, cap):
+@pytest.mark.parametrize("chunked", [False, True])
+def test_memory_cell_kernels_alone(H, dk, dv, cap, chunked):
     """Three sequences of unequal length in one launch, then a second launch that goes on
     from the state the first one left, in other slots than their order."""
     from gpt_fast_amd.ops import matrix_memory as M
     torch.manual_seed(H * 100 + dk)
     rows = M.RowLayout.fused(H, dk, dv)
-    lens1, lens2 = [5, 1, 37], [1, 9, 2]
+    if chunked and dk > 128:
+        pytest.skip("the chunked kernel takes key sizes up to 128")
+    # chunks of 32 tokens: runs of less than one, exactly one and two, and several with a rest
+    lens1, lens2 = ([5, 1, 37], [1, 9, 2]) if not chunked else ([5, 32, 137], [64, 9, 33])
     slots = [4, 0, 2]
     state = torch.zeros(6, M.state_size(H, dk, dv), device=DEV)
     state[1].fill_(7.0)                                        # a slot nobody uses stays as it is
@@ -112,7 +116,7 @@ def test_memory_cell_kernels_alone(H, dk, dv, cap):
         proj = torch.cat(chunks).contiguous()
         q_start = torch.tensor([sum(lens[:b]) for b in range(len(lens) + 1)], dtype=torch.int32, device=DEV)
         o = M.scan(proj, rows, bias, state, q_start, torch.tensor(slots, dtype=torch.int32, device=DEV),
-                   3, H, dk, dv, dk ** -0.5, cap or 0.0, 1e-6)
+                   3, H, dk, dv, dk ** -0.5, cap or 0.0, 1e-6, chunked=chunked)
         y = M.head_norm_gate(o, weight, proj, rows, 1e-5, torch.float32)
         at = 0
         for b, l in enumerate(lens):
