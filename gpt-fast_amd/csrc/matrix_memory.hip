@@ -162,10 +162,12 @@ extern "C" int gfa_matrix_memory_scan(const float* proj, const float* gate_bias,
 #define MC_COLS 32
 #define MC_PS (MC_L + 1)
 
-__host__ __device__ inline int mc_row_stride(int dk) {
-    const int dk4 = (dk + 3) / 4 * 4;
-    return (dk4 / 4) % 2 == 0 ? dk4 + 4 : dk4;      // in floats; a quarter of it is odd
-}
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float mc_floatx4_t;
+
+// rows of q and k in shared memory: dk filled up to a multiple of 16 (the matrix cores' tiles)
+// plus four floats, so that the sixteen rows a load touches lie in different banks
+__host__ __device__ inline int mc_padded(int dk) { return (dk + 15) / 16 * 16; }
+__host__ __device__ inline int mc_row_stride(int dk) { return mc_padded(dk) + 4; }
 
 __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
         const float* __restrict__ proj, const float* __restrict__ gate_bias,
@@ -173,16 +175,18 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
         const int* __restrict__ slots, float* __restrict__ out, MMShape s) {
     extern __shared__ __attribute__((aligned(16))) float mc_lds[];
     const int KS = mc_row_stride(s.dk);
-    const int dk4 = (s.dk + 3) / 4 * 4;
+    const int dkp = mc_padded(s.dk);
     float* Qs = mc_lds;                          // [MC_L][KS]
     float* Ks = Qs + MC_L * KS;                  // [MC_L][KS]
     float* Vs = Ks + MC_L * KS;                  // [MC_L][MC_COLS]
     float* Ps = Vs + MC_L * MC_COLS;             // [MC_L][MC_PS]
-    float* Ss = Ps + MC_L * MC_PS;               // [dk4][MC_COLS]
-    float* ns = Ss + dk4 * MC_COLS;              // [dk4]
-    float* gs = ns + dk4;                        // [MC_L] g_s
+    float* Ss = Ps + MC_L * MC_PS;               // [dkp][MC_COLS]
+    float* ns = Ss + dkp * MC_COLS;              // [dkp]
+    float* gs = ns + dkp;                        // [MC_L] g_s
     float* Ms = gs + MC_L;                       // [MC_L] M_t
     float* mt = Ms + MC_L;                       // [MC_L] m_t
+    float* ws = mt + MC_L;                       // [MC_L] exp(g_s - M of the chunk's last token)
+    float* nqs = ws + MC_L;                      // [MC_L] n_t . q_t
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col0 = blockIdx.x * MC_COLS;
     const int h = blockIdx.y, b = blockIdx.z;
@@ -193,37 +197,96 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
     float* const mptr = base + (size_t)s.H * s.dk * (s.dv + 1) + h;
     const float ib = gate_bias[h], fb = gate_bias[s.H + h];
 
-    for (int e = tid; e < dk4 * MC_COLS; e += 256) {
+    for (int e = tid; e < dkp * MC_COLS; e += 256) {
         const int d = e / MC_COLS, c = e % MC_COLS;
         Ss[e] = (d < s.dk && col0 + c < s.dv) ? S[(size_t)d * s.dv + col0 + c] : 0.f;
     }
-    for (int d = tid; d < dk4; d += 256) ns[d] = d < s.dk ? nvec[d] : 0.f;
+    for (int d = tid; d < dkp; d += 256) ns[d] = d < s.dk ? nvec[d] : 0.f;
+    for (int e = tid; e < 2 * MC_L * KS; e += 256) Qs[e] = 0.f;      // q and k: the filling stays zero
     float m_prev = *mptr;
+
+    // The rows of a chunk come from memory a chunk ahead: they are asked for before the chunk
+    // in hand is worked on and put into shared memory when it is done.  Rows whose q, k and v
+    // start at multiples of four floats travel as float4, four of q and k and one of v per
+    // thread (dk <= 128); other shapes element by element, without the look-ahead.
+    const int kq4 = s.dk / 4;
+    const bool vec = s.dk % 4 == 0 && s.dv % 4 == 0 && s.row_width % 4 == 0 && s.q_off % 4 == 0
+                     && s.k_off % 4 == 0 && s.v_off % 4 == 0;
+    float4 rq[4], rk[4], rv;
+    float ri = 0.f, rf = 0.f;
+    auto fetch = [&](int c0) {
+        const int Lc = t1 - c0 < MC_L ? t1 - c0 : MC_L;
+        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = tid + 256 * i, t = e / kq4, d4 = e - t * kq4;
+            rq[i] = rk[i] = zero;
+            if (t < Lc) {
+                const float* row = proj + (size_t)(c0 + t) * s.row_width + h * s.dk + d4 * 4;
+                rq[i] = *(const float4*)(row + s.q_off);
+                rk[i] = *(const float4*)(row + s.k_off);
+            }
+        }
+        {
+            const int t = tid >> 3, c4 = (tid & 7) * 4;
+            rv = zero;
+            if (t < Lc && col0 + c4 < s.dv)
+                rv = *(const float4*)(proj + (size_t)(c0 + t) * s.row_width + s.v_off + h * s.dv + col0 + c4);
+        }
+        if (wave == 0 && lane < Lc) {
+            const float* row = proj + (size_t)(c0 + lane) * s.row_width;
+            ri = row[s.i_off + h];
+            rf = row[s.f_off + h];
+        }
+    };
+    if (vec && t0 < t1) fetch(t0);
 
     for (int c0 = t0; c0 < t1; c0 += MC_L) {
         const int Lc = t1 - c0 < MC_L ? t1 - c0 : MC_L;
         __syncthreads();                         // the chunk before is done with Qs .. Ss
-        // q (scaled), k, v of the chunk; rows beyond its end and columns beyond dk are zero
-        for (int e = tid; e < MC_L * KS; e += 256) {
-            const int t = e / KS, d = e - t * KS;
-            const bool ok = t < Lc && d < s.dk;
-            const float* row = proj + (size_t)(c0 + t) * s.row_width;
-            Qs[e] = ok ? row[s.q_off + h * s.dk + d] * s.q_scale : 0.f;
-            Ks[e] = ok ? row[s.k_off + h * s.dk + d] : 0.f;
-        }
-        for (int e = tid; e < MC_L * MC_COLS; e += 256) {
-            const int t = e / MC_COLS, c = e % MC_COLS;
-            Vs[e] = (t < Lc && col0 + c < s.dv)
-                ? proj[(size_t)(c0 + t) * s.row_width + s.v_off + h * s.dv + col0 + c] : 0.f;
+        float ipre = 0.f, fpre = 0.f;
+        if (vec) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int e = tid + 256 * i, t = e / kq4, d4 = e - t * kq4;
+                if (t < MC_L) {
+                    float4 x = rq[i];
+                    x.x *= s.q_scale; x.y *= s.q_scale; x.z *= s.q_scale; x.w *= s.q_scale;
+                    *(float4*)(Qs + t * KS + d4 * 4) = x;
+                    *(float4*)(Ks + t * KS + d4 * 4) = rk[i];
+                }
+            }
+            *(float4*)(Vs + (tid >> 3) * MC_COLS + (tid & 7) * 4) = rv;
+            ipre = ri;
+            fpre = rf;
+            if (c0 + MC_L < t1) fetch(c0 + MC_L);
+        } else {
+            // q (scaled), k, v of the chunk; rows beyond its end and columns beyond dk are zero
+            for (int e = tid; e < MC_L * KS; e += 256) {
+                const int t = e / KS, d = e - t * KS;
+                const bool ok = t < Lc && d < s.dk;
+                const float* row = proj + (size_t)(c0 + t) * s.row_width;
+                Qs[e] = ok ? row[s.q_off + h * s.dk + d] * s.q_scale : 0.f;
+                Ks[e] = ok ? row[s.k_off + h * s.dk + d] : 0.f;
+            }
+            for (int e = tid; e < MC_L * MC_COLS; e += 256) {
+                const int t = e / MC_COLS, c = e % MC_COLS;
+                Vs[e] = (t < Lc && col0 + c < s.dv)
+                    ? proj[(size_t)(c0 + t) * s.row_width + s.v_off + h * s.dv + col0 + c] : 0.f;
+            }
+            if (wave == 0 && lane < Lc) {
+                const float* row = proj + (size_t)(c0 + lane) * s.row_width;
+                ipre = row[s.i_off + h];
+                fpre = row[s.f_off + h];
+            }
         }
         if (wave == 0) {
             // the gates of the chunk: running sum of f, running maximum of g, one token per lane
             const int t = lane;
             float ig = -INFINITY, fg = 0.f;
             if (t < Lc) {
-                const float* row = proj + (size_t)(c0 + t) * s.row_width;
-                ig = mm_cap(row[s.i_off + h] + ib, s.cap);
-                fg = mm_logsigmoid(mm_cap(row[s.f_off + h] + fb, s.cap));
+                ig = mm_cap(ipre + ib, s.cap);
+                fg = mm_logsigmoid(mm_cap(fpre + fb, s.cap));
             }
             float F = fg;
 #pragma unroll
@@ -238,103 +301,101 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
                 const float up = __shfl_up(M, o, GFA_WAVE);
                 if (lane >= o) M = fmaxf(M, up);
             }
+            const float M_last = __shfl(M, Lc - 1, GFA_WAVE);
             if (t < MC_L) {
                 gs[t] = g;
                 Ms[t] = M;
                 mt[t] = F + M;
+                ws[t] = expf(g - M_last);
             }
         }
         __syncthreads();
+        // The products run on the matrix cores in float (v_mfma_f32_16x16x4_f32: lane l
+        // supplies A[l % 16][l / 16] and B[l / 16][l % 16] and holds C[4 (l / 16) .. +3][l % 16]),
+        // a 16 x 16 tile of the result per wave and loop.
+        const int li = lane & 15, lg = lane >> 4;
         // scores of the chunk, weighted: P[t][s] = (q_t . k_s) exp(g_s - M_t) for s <= t
         {
-            const int ty = tid >> 4, tx = tid & 15;
-            float a00 = 0.f, a01 = 0.f, a10 = 0.f, a11 = 0.f;
-            const float4* q0 = (const float4*)(Qs + ty * KS);
-            const float4* q1 = (const float4*)(Qs + (ty + 16) * KS);
-            const float4* k0 = (const float4*)(Ks + tx * KS);
-            const float4* k1 = (const float4*)(Ks + (tx + 16) * KS);
-            for (int d = 0; d < dk4 / 4; ++d) {
-                const float4 x0 = q0[d], x1 = q1[d], y0 = k0[d], y1 = k1[d];
-                a00 = fmaf(x0.x, y0.x, fmaf(x0.y, y0.y, fmaf(x0.z, y0.z, fmaf(x0.w, y0.w, a00))));
-                a01 = fmaf(x0.x, y1.x, fmaf(x0.y, y1.y, fmaf(x0.z, y1.z, fmaf(x0.w, y1.w, a01))));
-                a10 = fmaf(x1.x, y0.x, fmaf(x1.y, y0.y, fmaf(x1.z, y0.z, fmaf(x1.w, y0.w, a10))));
-                a11 = fmaf(x1.x, y1.x, fmaf(x1.y, y1.y, fmaf(x1.z, y1.z, fmaf(x1.w, y1.w, a11))));
+            const int ti = wave >> 1, si = wave & 1;
+            mc_floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+            if (si <= ti) {                       // the tile above the diagonal is all zero
+                const float* qa = Qs + (ti * 16 + li) * KS + lg;
+                const float* kb = Ks + (si * 16 + li) * KS + lg;
+                for (int d0 = 0; d0 < dkp; d0 += 4)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[d0], kb[d0], acc, 0, 0, 0);
             }
-            auto weight = [&](int t, int ss, float a) {
-                return ss <= t ? a * expf(gs[ss] - Ms[t]) : 0.f;    // g of a missing token is -inf
-            };
-            Ps[ty * MC_PS + tx] = weight(ty, tx, a00);
-            Ps[ty * MC_PS + tx + 16] = weight(ty, tx + 16, a01);
-            Ps[(ty + 16) * MC_PS + tx] = weight(ty + 16, tx, a10);
-            Ps[(ty + 16) * MC_PS + tx + 16] = weight(ty + 16, tx + 16, a11);
+            const int ss = si * 16 + li;
+            const float g = gs[ss];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = ti * 16 + lg * 4 + r;
+                Ps[t * MC_PS + ss] = ss <= t ? acc[r] * expf(g - Ms[t]) : 0.f;   // g of a missing token is -inf
+            }
         }
         __syncthreads();
-        // o_t for the workgroup's columns: four columns per thread, eight threads per token
+        // n_t . q_t: eight threads per token
         {
-            const int t = tid >> 3, j = tid & 7, c4 = j * 4;
-            const float carry = expf(m_prev - Ms[t]);
-            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+            const int t = tid >> 3, j = tid & 7;
             const float* qr = Qs + t * KS;
-            for (int d = 0; d < s.dk; ++d) {
-                const float x = qr[d];
-                const float4 sv = *(const float4*)(Ss + d * MC_COLS + c4);
-                acc.x = fmaf(x, sv.x, acc.x);
-                acc.y = fmaf(x, sv.y, acc.y);
-                acc.z = fmaf(x, sv.z, acc.z);
-                acc.w = fmaf(x, sv.w, acc.w);
-            }
-            acc.x *= carry; acc.y *= carry; acc.z *= carry; acc.w *= carry;
             const float* pr = Ps + t * MC_PS;
-            for (int ss = 0; ss <= t; ++ss) {
-                const float x = pr[ss];
-                const float4 vv = *(const float4*)(Vs + ss * MC_COLS + c4);
-                acc.x = fmaf(x, vv.x, acc.x);
-                acc.y = fmaf(x, vv.y, acc.y);
-                acc.z = fmaf(x, vv.z, acc.z);
-                acc.w = fmaf(x, vv.w, acc.w);
-            }
             float nq0 = 0.f, nq1 = 0.f;
             for (int d = j; d < s.dk; d += 8) nq0 = fmaf(qr[d], ns[d], nq0);
             for (int ss = j; ss <= t; ss += 8) nq1 += pr[ss];
-            float nq = carry * nq0 + nq1;
+            float nq = expf(m_prev - Ms[t]) * nq0 + nq1;
             nq += __shfl_xor(nq, 1, GFA_WAVE);
             nq += __shfl_xor(nq, 2, GFA_WAVE);
             nq += __shfl_xor(nq, 4, GFA_WAVE);
-            if (t < Lc) {
-                const float inv = 1.f / (fmaxf(fabsf(nq), expf(-mt[t])) + s.den_eps);
-                float* dst = out + (size_t)(c0 + t) * s.H * s.dv + (size_t)h * s.dv + col0 + c4;
-                const float r[4] = {acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv};
+            if (j == 0) nqs[t] = nq;
+        }
+        // o_t for the workgroup's columns: exp(m0 - M_t) (Q S0) + P V
+        mc_floatx4_t num;
+        const int oti = wave >> 1, oci = wave & 1;
+        {
+            num = mc_floatx4_t{0.f, 0.f, 0.f, 0.f};
+            const float* qa = Qs + (oti * 16 + li) * KS + lg;
+            const float* sb = Ss + lg * MC_COLS + oci * 16 + li;
+            for (int d0 = 0; d0 < dkp; d0 += 4)
+                num = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[d0], sb[d0 * MC_COLS], num, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (col0 + c4 + i < s.dv) dst[i] = r[i];
+            for (int r = 0; r < 4; ++r) num[r] *= expf(m_prev - Ms[oti * 16 + lg * 4 + r]);
+            const float* pa = Ps + (oti * 16 + li) * MC_PS + lg;
+            const float* vb = Vs + lg * MC_COLS + oci * 16 + li;
+            for (int s0 = 0; s0 < (oti + 1) * 16; s0 += 4)
+                num = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[s0], vb[s0 * MC_COLS], num, 0, 0, 0);
+        }
+        __syncthreads();                         // nqs is written; Ss has been read by every wave
+        {
+            const int c = col0 + oci * 16 + li;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = oti * 16 + lg * 4 + r;
+                if (t < Lc && c < s.dv) {
+                    const float den = fmaxf(fabsf(nqs[t]), expf(-mt[t])) + s.den_eps;
+                    out[(size_t)(c0 + t) * s.H * s.dv + (size_t)h * s.dv + c] = num[r] / den;
+                }
             }
         }
-        __syncthreads();
-        // the state after the chunk's last token
+        // the state after the chunk's last token: S = decay S + (w K)^T V, a wave's tiles of 16
+        // rows of S by 16 columns in turn
         {
-            const float M_end = Ms[Lc - 1];
-            const float decay = expf(m_prev - M_end);
-            const int dr = tid >> 3, c4 = (tid & 7) * 4;
+            const float decay = expf(m_prev - Ms[Lc - 1]);
+            for (int tile = wave; tile < (dkp / 16) * 2; tile += 4) {
+                const int di = tile >> 1, ci = tile & 1;
+                float* sc = Ss + (di * 16 + lg * 4) * MC_COLS + ci * 16 + li;
+                mc_floatx4_t acc;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int d = dr + 32 * i;
-                if (d < s.dk) {
-                    float4 acc = *(const float4*)(Ss + d * MC_COLS + c4);
-                    acc.x *= decay; acc.y *= decay; acc.z *= decay; acc.w *= decay;
-                    for (int ss = 0; ss < Lc; ++ss) {
-                        const float x = expf(gs[ss] - M_end) * Ks[ss * KS + d];
-                        const float4 vv = *(const float4*)(Vs + ss * MC_COLS + c4);
-                        acc.x = fmaf(x, vv.x, acc.x);
-                        acc.y = fmaf(x, vv.y, acc.y);
-                        acc.z = fmaf(x, vv.z, acc.z);
-                        acc.w = fmaf(x, vv.w, acc.w);
-                    }
-                    *(float4*)(Ss + d * MC_COLS + c4) = acc;
-                }
+                for (int r = 0; r < 4; ++r) acc[r] = decay * sc[r * MC_COLS];
+                const float* ka = Ks + lg * KS + di * 16 + li;
+                const float* vb = Vs + lg * MC_COLS + ci * 16 + li;
+                for (int s0 = 0; s0 < MC_L; s0 += 4)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ws[s0 + lg] * ka[s0 * KS], vb[s0 * MC_COLS],
+                                                              acc, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sc[r * MC_COLS] = acc[r];
             }
             for (int d = tid; d < s.dk; d += 256) {
                 float a = decay * ns[d];
-                for (int ss = 0; ss < Lc; ++ss) a = fmaf(expf(gs[ss] - M_end), Ks[ss * KS + d], a);
+                for (int ss = 0; ss < Lc; ++ss) a = fmaf(ws[ss], Ks[ss * KS + d], a);
                 ns[d] = a;
             }
             m_prev = mt[Lc - 1];
@@ -352,9 +413,9 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
 }
 
 extern "C" int gfa_matrix_memory_chunk_lds(int dk) {
-    const int dk4 = (dk + 3) / 4 * 4;
+    const int dkp = mc_padded(dk);
     return (int)sizeof(float) * (2 * MC_L * mc_row_stride(dk) + MC_L * MC_COLS + MC_L * MC_PS
-                                 + dk4 * MC_COLS + dk4 + 3 * MC_L);
+                                 + dkp * MC_COLS + dkp + 5 * MC_L);
 }
 
 extern "C" int gfa_matrix_memory_chunks(const float* proj, const float* gate_bias, float* state,
