@@ -321,6 +321,7 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
             if (si <= ti) {                       // the tile above the diagonal is all zero
                 const float* qa = Qs + (ti * 16 + li) * KS + lg;
                 const float* kb = Ks + (si * 16 + li) * KS + lg;
+#pragma unroll 4
                 for (int d0 = 0; d0 < dkp; d0 += 4)
                     acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[d0], kb[d0], acc, 0, 0, 0);
             }
@@ -354,12 +355,14 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
             num = mc_floatx4_t{0.f, 0.f, 0.f, 0.f};
             const float* qa = Qs + (oti * 16 + li) * KS + lg;
             const float* sb = Ss + lg * MC_COLS + oci * 16 + li;
+#pragma unroll 4
             for (int d0 = 0; d0 < dkp; d0 += 4)
                 num = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[d0], sb[d0 * MC_COLS], num, 0, 0, 0);
 #pragma unroll
             for (int r = 0; r < 4; ++r) num[r] *= expf(m_prev - Ms[oti * 16 + lg * 4 + r]);
             const float* pa = Ps + (oti * 16 + li) * MC_PS + lg;
             const float* vb = Vs + lg * MC_COLS + oci * 16 + li;
+#pragma unroll 4
             for (int s0 = 0; s0 < (oti + 1) * 16; s0 += 4)
                 num = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[s0], vb[s0 * MC_COLS], num, 0, 0, 0);
         }
@@ -387,6 +390,7 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
                 for (int r = 0; r < 4; ++r) acc[r] = decay * sc[r * MC_COLS];
                 const float* ka = Ks + lg * KS + di * 16 + li;
                 const float* vb = Vs + lg * MC_COLS + ci * 16 + li;
+#pragma unroll
                 for (int s0 = 0; s0 < MC_L; s0 += 4)
                     acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ws[s0 + lg] * ka[s0 * KS], vb[s0 * MC_COLS],
                                                               acc, 0, 0, 0);

@@ -19,8 +19,11 @@ from typing import Dict
 
 import torch
 
+from ..ops.kernels import PAGE
 from .batch import Entry
 from .step import Engine
+
+SPARE_SEQUENCES = 64
 
 
 def replay(engine: Engine, lines, out_dir: str, log=None) -> int:
@@ -68,10 +71,13 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time, each rounded up to 64")
+                    help="most tokens live requests hold at any time; the cache is sized for them "
+                         "and for the pages that requests leave partly filled")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
+    # a request holds whole pages: room for the tokens, and for a partly filled page of each of
+    # as many requests as SPARE_SEQUENCES
     engine = Engine.from_folder(args.model, dtype=args.dtype, device=args.device,
-                                max_tokens=args.max_tokens)
+                                max_tokens=args.max_tokens + PAGE * SPARE_SEQUENCES)
     replay(engine, sys.stdin, args.out)
     return 0

@@ -50,6 +50,10 @@ class Engine:
     def from_plan(cls, plan, parameters, dtype, device="cuda:0", **cache_args) -> "Engine":
         rt = Runtime(compute_dtype(dtype), _device(device))
         model = DecoderModel(plan, rt)
+        # the HIP libraries this model's steps call, built together if any is missing (each
+        # would else be built alone at its first call)
+        from ..csrc import build as _build
+        _build.ensure([n for n in model.kernel_libraries() if n in _build.available_modules()])
         model.bind(parameters)
         return cls(model, **cache_args)
 

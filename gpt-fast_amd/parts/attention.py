@@ -61,6 +61,10 @@ class Attention(Part):
         s = self.spec
         return (s.n_heads + 2 * s.n_kv_heads) * s.head_dim
 
+    @staticmethod
+    def libraries(runtime):
+        return () if runtime.is_float32 else ("attention_bf16",)
+
     defers_sum = True              # ``residual`` may be a parts.base.ResidualStream
     takes_prepared = True          # x may be an ops.linear.HalfNormed
 

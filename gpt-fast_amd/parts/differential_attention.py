@@ -22,6 +22,7 @@ class DifferentialAttention(Part):
     then ``wo``.  The projections of q, k, v and the gate are one matrix ``w_in``.  Scores,
     softmax, sums, the combination and the norm are float32."""
 
+    libraries = ("differential_attention",)
     defers_sum = True              # ``residual`` may be a parts.base.ResidualStream
     takes_prepared = True          # x may be an ops.linear.HalfNormed
 

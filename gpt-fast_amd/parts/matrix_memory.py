@@ -26,6 +26,7 @@ class MatrixMemory(Part):
     at the operand of ``wo``."""
 
     replayable = True
+    libraries = ("matrix_memory",)
     defers_sum = True              # ``residual`` may be a parts.base.ResidualStream
     takes_prepared = True          # x may be an ops.linear.HalfNormed
 

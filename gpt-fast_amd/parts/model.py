@@ -118,6 +118,26 @@ class DecoderModel:
             flops += getattr(block, "step_flops", lambda q, s: 0.0)(q_lens, starts)
         return flops
 
+    def kernel_libraries(self):
+        """Names of the compiled libraries (csrc/<name>.hip) that a step of this model calls:
+        the ones every model uses, by the engine's type, and those its parts name in
+        ``libraries`` (a tuple, or a function of the runtime)."""
+        names = ["core"]
+        if not self.rt.is_float32:
+            names += ["gemm_bf16", "gemm_wide_bf16", "gemm_tiled_bf16"]
+
+        def visit(part):
+            libs = getattr(part, "libraries", ())
+            for n in (libs(self.rt) if callable(libs) else libs):
+                if n not in names:
+                    names.append(n)
+            for child in getattr(part, "children", lambda: {})().values():
+                visit(child)
+        for part in list(self.blocks) + [self.final_norm, self.input_position]:
+            if part is not None:
+                visit(part)
+        return names
+
     def step_fields(self):
         """The further fields of a step's description that the parts ask for, each once (by
         name: layers of one kind ask for the same field)."""
