@@ -156,8 +156,8 @@ class PigodraConfig:
     # ------------------------------------------------------------------ named shapes
     @staticmethod
     def from_name(name: str) -> "PigodraConfig":
-        """Shapes for measurements (random weights): ``pigodra-<width>`` with a width in
-        PRESET_WIDTHS; 128-wide heads, three matrix-memory layers to one attention layer."""
+        """Shapes for measurements (random weights): ``pigodra-<width>``; heads of 128, three
+        matrix-memory layers to one attention layer, a feed-forward in every layer."""
         key = name.lower()
         if key not in PRESETS:
             raise KeyError(f"no Pigodra preset '{name}'; known: {sorted(PRESETS)}")
@@ -182,8 +182,8 @@ def _stack(width: int, n_layers: int, ff: int, kv_heads: int, vocab: int = 32000
 
 
 PRESETS = {
-    # the widths of a 1B- and an 8B-class dense decoder (the latter is the shape of the
-    # library's Llama-3.1-8B preset: width 4096, inner size 14336, 32 heads of 128, 8 kv heads)
-    "pigodra-2048": lambda: _stack(2048, 16, 8192, 8),
+    # the widths, inner sizes, head sizes and vocabularies of the library's llama-3.1-8b and
+    # llama-3.1-70b presets: the same rows of q, k, v and output per layer
     "pigodra-4096": lambda: _stack(4096, 32, 14336, 8, vocab=128256),
+    "pigodra-8192": lambda: _stack(8192, 80, 28672, 8, vocab=128256),
 }

@@ -12,7 +12,7 @@
 //
 // Epilogues (MODE): 0 store bfloat16, 1 store float, 2 add into a float matrix (the
 // residual stream), 3 gate: out[m, n] = silu(x W[n]) * (x W[n + gate_rows]) in bfloat16
-// (the reference's feed-forward, model.py:227).
+// (the reference's feed-forward, model.py:227), 6 the same gate with the tanh form of gelu.
 #include "common.h"
 
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
@@ -28,14 +28,21 @@ __device__ __forceinline__ float dot8(const Pack8& a, const Pack8& b, float acc)
     return acc;
 }
 
-__device__ __forceinline__ float silu(float a) { return a / (1.f + expf(-a)); }
+// MODE 3 gates with silu, MODE 6 with the tanh form of gelu; everything else about the two is
+// the same
+#define IS_GATE(M) ((M) == 3 || (M) == 6)
+template <int MODE>
+__device__ __forceinline__ float gate_act(float a) {
+    if (MODE == 6) return 0.5f * a * (1.f + tanhf(0.7978845608028654f * (a + 0.044715f * a * a * a)));
+    return a / (1.f + expf(-a));
+}
 
 template <int MODE>
 __device__ __forceinline__ void skinny_store(void* out, int ldo, int m, int n, float v, float gate_v,
                                              int out_pad = 0) {
     if (MODE == 4) return;                     // the rotary epilogue stores by itself
-    if (MODE == 3 && out_pad) {
-        ((bf16_t*)out)[chunked_elem(m, n, out_pad)] = float_to_bf16(silu(v) * gate_v);
+    if (IS_GATE(MODE) && out_pad) {
+        ((bf16_t*)out)[chunked_elem(m, n, out_pad)] = float_to_bf16(gate_act<MODE>(v) * gate_v);
         return;
     }
     if (MODE == 0) {
@@ -46,7 +53,7 @@ __device__ __forceinline__ void skinny_store(void* out, int ldo, int m, int n, f
         float* o = (float*)out + (size_t)m * ldo + n;
         *o = *o + v;
     } else {
-        ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(silu(v) * gate_v);
+        ((bf16_t*)out)[(size_t)m * ldo + n] = float_to_bf16(gate_act<MODE>(v) * gate_v);
     }
 }
 
@@ -79,7 +86,7 @@ __global__ __launch_bounds__(256) void skinny_dot_kernel(
         int N, int K, int ldo, int gate_rows, int kc) {
     extern __shared__ uint4 xs[];                      // [MT][kc / 8]
     constexpr int WR = 4;
-    constexpr int COLS = (MODE == 3) ? 2 : 4;
+    constexpr int COLS = (IS_GATE(MODE)) ? 2 : 4;
     const int lane = threadIdx.x & 63;
     const int n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * COLS;
     const bool active = n0 < N;
@@ -88,9 +95,9 @@ __global__ __launch_bounds__(256) void skinny_dot_kernel(
     const bf16_t* wrow[WR];
 #pragma unroll
     for (int r = 0; r < WR; ++r) {
-        int n = n0 + (MODE == 3 ? (r & 1) : r);
+        int n = n0 + (IS_GATE(MODE) ? (r & 1) : r);
         if (n >= N) n = N - 1;                         // clamped rows are computed, not stored
-        if (MODE == 3 && r >= 2) n += gate_rows;
+        if (IS_GATE(MODE) && r >= 2) n += gate_rows;
         wrow[r] = w + (size_t)n * K;
     }
     float acc[WR * MT];
@@ -145,7 +152,7 @@ __global__ __launch_bounds__(256) void skinny_dot_kernel(
     constexpr int GROUP = 64 / (WR * MT);
     float total = acc[0];
     float gate_v = 0.f;
-    if (MODE == 3) gate_v = __shfl(total, (lane + 32) & 63, GFA_WAVE);   // value v + 2 MT
+    if (IS_GATE(MODE)) gate_v = __shfl(total, (lane + 32) & 63, GFA_WAVE);   // value v + 2 MT
     const int v = lane / GROUP;
     const int r = v / MT, m = v - r * MT;
     if (lane % GROUP == 0 && r < COLS && m < M && n0 + r < N)
@@ -165,10 +172,10 @@ __global__ __launch_bounds__(256) void skinny_scalar_kernel(
         for (int k = lane; k < K; k += 64) {
             const float xv = bf16_to_float(x[(size_t)m * K + k]);
             a = fmaf(xv, bf16_to_float(w[(size_t)n * K + k]), a);
-            if (MODE == 3) b = fmaf(xv, bf16_to_float(w[(size_t)(n + gate_rows) * K + k]), b);
+            if (IS_GATE(MODE)) b = fmaf(xv, bf16_to_float(w[(size_t)(n + gate_rows) * K + k]), b);
         }
         a = wave_sum(a);
-        if (MODE == 3) b = wave_sum(b);
+        if (IS_GATE(MODE)) b = wave_sum(b);
         if (lane == 0) skinny_store<MODE>(out, ldo, m, n, a, b);
     }
 }
@@ -176,7 +183,7 @@ __global__ __launch_bounds__(256) void skinny_scalar_kernel(
 template <int MODE>
 static int launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K,
                          int ldo, int gate_rows, hipStream_t stream) {
-    const size_t out_elem = (MODE == 0 || MODE == 3) ? sizeof(bf16_t) : sizeof(float);
+    const size_t out_elem = (MODE == 0 || IS_GATE(MODE)) ? sizeof(bf16_t) : sizeof(float);
     if (K % 8 != 0) {
         for (int m0 = 0; m0 < M; m0 += 16) {
             const int mc = (M - m0 < 16) ? M - m0 : 16;
@@ -190,7 +197,7 @@ static int launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int M, int
         const int mc = (M - m0 < 8) ? M - m0 : 8;
         const bf16_t* xs = x + (size_t)m0 * K;
         void* os = (char*)out + (size_t)m0 * ldo * out_elem;
-        constexpr int COLS = (MODE == 3) ? 2 : 4;
+        constexpr int COLS = (IS_GATE(MODE)) ? 2 : 4;
         const int blocks = (N + 4 * COLS - 1) / (4 * COLS);
         const int mt = mc == 1 ? 1 : mc == 2 ? 2 : mc <= 4 ? 4 : 8;
         int kc = (65536 / (mt * 2)) & ~511;            // 64 KiB of x per workgroup
@@ -279,8 +286,8 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
         const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M,
         int N, int K, int ldo, int gate_rows, int th, SkinnyExtra ex) {
     static_assert(TILES == 1 || (TILES == 2 && CT <= 3 && MODE != 3), "two tiles: up to 48 rows of x, no gate");
-    constexpr int RT = (MODE == 3) ? 2 : TILES;          // tiles of W's rows multiplied per x fragment
-    constexpr int NT = (MODE == 3) ? 1 : TILES;          // tiles of output columns per workgroup
+    constexpr int RT = (IS_GATE(MODE)) ? 2 : TILES;          // tiles of W's rows multiplied per x fragment
+    constexpr int NT = (IS_GATE(MODE)) ? 1 : TILES;          // tiles of output columns per workgroup
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, NW = blockDim.x >> 6;
     // th (12..16) rows of W per tile: the host picks it so that the tiles divide evenly
@@ -307,9 +314,9 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int r = lrow + 4 * j;
-            int n = n0 + (MODE == 3 ? 0 : rt * th) + (r < th ? r : th - 1);
+            int n = n0 + (IS_GATE(MODE) ? 0 : rt * th) + (r < th ? r : th - 1);
             if (n >= N) n = N - 1;                       // clamped rows are computed, not stored
-            wsrc[rt][j] = w + (size_t)(n + (MODE == 3 ? rt * gate_rows : 0)) * K + lchunk * 8;
+            wsrc[rt][j] = w + (size_t)(n + (IS_GATE(MODE) ? rt * gate_rows : 0)) * K + lchunk * 8;
         }
     // two register sets: while piece t is multiplied, pieces t + 1 and t + 2 are in flight
     uint4 regs_a[RT][4], regs_b[RT][4];
@@ -650,7 +657,7 @@ __global__ __launch_bounds__(512) void skinny_mfma_kernel(
             for (int j = 0; j < 4; ++j) {
                 const int n = nb + fg * 4 + j;
                 if (n < N && fg * 4 + j < th)
-                    skinny_store<MODE>(out, ldo, m, n, acc[ot][ct][j], MODE == 3 ? acc[RT - 1][ct][j] : 0.f, ex.out_pad);
+                    skinny_store<MODE>(out, ldo, m, n, acc[ot][ct][j], IS_GATE(MODE) ? acc[RT - 1][ct][j] : 0.f, ex.out_pad);
             }
         }
     }
@@ -715,7 +722,7 @@ static int pick_tile_rows(int N, int step, int nt = 1) {
 static int tiles_per_workgroup(int mode, int M, int N) {
     // 33..48 rows: only where the registers hold it (the plain epilogues)
     const int most = (mode == 2 || mode == 4) ? 32 : 48;
-    return (mode != 3 && M > 8 && M <= most && N >= 24 * compute_units()) ? 2 : 1;
+    return (!IS_GATE(mode) && M > 8 && M <= most && N >= 24 * compute_units()) ? 2 : 1;
 }
 
 // Tile height the launcher below uses for this mode, these rows of x and this width.
@@ -740,10 +747,10 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
     const int nt = tiles_per_workgroup(MODE, M, N);
     const int th = ct == 1 ? tile_rows(MODE, M, N) : 16;
     const int tiles = (N + th * nt - 1) / (th * nt);     // workgroups
-    const int RT = (MODE == 3) ? 2 : nt;                 // tiles of W staged per wave
+    const int RT = (IS_GATE(MODE)) ? 2 : nt;                 // tiles of W staged per wave
     const int pieces = (K + SM_SUBK - 1) / SM_SUBK;
     int nw = 1;                                          // waves per tile: aim at >= 2048 waves,
-    const int nw_max = (MODE == 3) ? 4 : 8;
+    const int nw_max = (IS_GATE(MODE)) ? 4 : 8;
     // at least four waves per tile where K allows: one wave walking sixteen rows alone
     // streams measurably slower than four that share them
     while (nw < nw_max && (tiles * nw < 2048 || nw < 4) && pieces >= 4 * nw) nw *= 2;
@@ -781,23 +788,23 @@ static int launch_skinny_mfma(const bf16_t* x, const bf16_t* w, void* out, int M
         case 1:                                          // columns of the x operand that stand
             if (M <= 4) GFA_LAUNCH_MFMA(1, 4, false, 1);   // for no row carry later steps of k
             else if (M <= 8) GFA_LAUNCH_MFMA(1, 2, false, 1);
-            else if (nt == 2) GFA_LAUNCH_MFMA(1, 1, true, (MODE == 3 ? 1 : 2));
+            else if (nt == 2) GFA_LAUNCH_MFMA(1, 1, true, (IS_GATE(MODE) ? 1 : 2));
             else GFA_LAUNCH_MFMA(1, 1, true, 1);
             break;
         case 2:                                          // 17..20, ..24 rows: a narrower second tile
             if (M <= 20) {
-                if (nt == 2) GFA_LAUNCH_MFMA_L(2, 1, false, (MODE == 3 ? 1 : 2), 4);
+                if (nt == 2) GFA_LAUNCH_MFMA_L(2, 1, false, (IS_GATE(MODE) ? 1 : 2), 4);
                 else GFA_LAUNCH_MFMA_L(2, 1, false, 1, 4);
             } else if (M <= 24) {
-                if (nt == 2) GFA_LAUNCH_MFMA_L(2, 1, false, (MODE == 3 ? 1 : 2), 2);
+                if (nt == 2) GFA_LAUNCH_MFMA_L(2, 1, false, (IS_GATE(MODE) ? 1 : 2), 2);
                 else GFA_LAUNCH_MFMA_L(2, 1, false, 1, 2);
             } else {
-                if (nt == 2) GFA_LAUNCH_MFMA(2, 1, false, (MODE == 3 ? 1 : 2));
+                if (nt == 2) GFA_LAUNCH_MFMA(2, 1, false, (IS_GATE(MODE) ? 1 : 2));
                 else GFA_LAUNCH_MFMA(2, 1, false, 1);
             }
             break;
         case 3:
-            if (nt == 2) GFA_LAUNCH_MFMA(3, 1, false, (MODE == 3 ? 1 : 2));
+            if (nt == 2) GFA_LAUNCH_MFMA(3, 1, false, (IS_GATE(MODE) ? 1 : 2));
             else GFA_LAUNCH_MFMA(3, 1, false, 1);
             break;
         default: GFA_LAUNCH_MFMA(4, 1, false, 1); break;
@@ -819,6 +826,7 @@ extern "C" int gfa_skinny_mfma_bf16(const void* x, const void* w, void* out, int
         case 1: return launch_skinny_mfma<1>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
         case 2: return launch_skinny_mfma<2>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
         case 3: return launch_skinny_mfma<3>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 6: return launch_skinny_mfma<6>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
     }
     return (int)hipErrorInvalidValue;
 }
@@ -891,7 +899,7 @@ extern "C" int gfa_skinny_after_chain_bf16(const void* xg, const float* ssq_in, 
                                            hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K <= 0 || K % 8 != 0 || !ssq_in || t_in <= 0) return (int)hipErrorInvalidValue;
-    if (out_chunked && (mode != 3 || N % 8 != 0)) return (int)hipErrorInvalidValue;
+    if (out_chunked && (!IS_GATE(mode) || N % 8 != 0)) return (int)hipErrorInvalidValue;
     SkinnyExtra ex = {};
     ex.ssq_in = ssq_in;
     ex.t_in = t_in;
@@ -905,6 +913,7 @@ extern "C" int gfa_skinny_after_chain_bf16(const void* xg, const float* ssq_in, 
         case 0: return launch_skinny_mfma<0>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
         case 1: return launch_skinny_mfma<1>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
         case 3: return launch_skinny_mfma<3>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
+        case 6: return launch_skinny_mfma<6>(xp, wp, out, M, N, K, ldo, gate_rows, ex, stream);
     }
     return (int)hipErrorInvalidValue;
 }
@@ -921,6 +930,7 @@ extern "C" int gfa_skinny_bf16(const void* x, const void* w, void* out, int M, i
         case 1: return launch_skinny<1>(xp, wp, out, M, N, K, ldo, gate_rows, stream);
         case 2: return launch_skinny<2>(xp, wp, out, M, N, K, ldo, gate_rows, stream);
         case 3: return launch_skinny<3>(xp, wp, out, M, N, K, ldo, gate_rows, stream);
+        case 6: return launch_skinny<6>(xp, wp, out, M, N, K, ldo, gate_rows, stream);
     }
     return (int)hipErrorInvalidValue;
 }

@@ -95,8 +95,18 @@ def skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     return out
 
 
-def skinny_gated(x: torch.Tensor, w13: torch.Tensor, out: Optional[torch.Tensor] = None):
-    """[M, I] = silu(x W1^T) * (x W3^T), w13 = [2I, K]: rows of W1, then rows of W3."""
+GATE_MODES = {"silu": 3, "gelu_tanh": 6}     # the kernels' epilogue numbers
+
+
+def _gate_mode(activation: str) -> int:
+    if activation not in GATE_MODES:
+        raise KernelError(f"gate activation '{activation}': {sorted(GATE_MODES)}")
+    return GATE_MODES[activation]
+
+
+def skinny_gated(x: torch.Tensor, w13: torch.Tensor, out: Optional[torch.Tensor] = None,
+                 activation: str = "silu"):
+    """[M, I] = act(x W1^T) * (x W3^T), w13 = [2I, K]: rows of W1, then rows of W3."""
     _check_operands(x, w13, "skinny_gated")
     M, K = x.shape
     if w13.shape[0] % 2:
@@ -106,8 +116,8 @@ def skinny_gated(x: torch.Tensor, w13: torch.Tensor, out: Optional[torch.Tensor]
         out = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
     elif out.shape != (M, I) or out.dtype != torch.bfloat16 or not out.is_contiguous():
         raise KernelError("skinny_gated: out has the wrong shape or dtype")
-    check(_entry(M, K)(ptr(x), ptr(w13), ptr(out), _i(M), _i(I), _i(K), _i(I), _i(3), _i(I),
-                       stream_handle()), "skinny_gated")
+    check(_entry(M, K)(ptr(x), ptr(w13), ptr(out), _i(M), _i(I), _i(K), _i(I),
+                       _i(_gate_mode(activation)), _i(I), stream_handle()), "skinny_gated")
     return out
 
 
@@ -179,8 +189,9 @@ def skinny_after_chain(xg, ssq, eps: float, w, out_dtype=torch.bfloat16):
     return out
 
 
-def skinny_after_chain_gated(xg, ssq, eps: float, w13, chunked: bool = False):
-    """silu(n W1^T) * (n W3^T) with n the normed rows given by their two halves; ``chunked``:
+def skinny_after_chain_gated(xg, ssq, eps: float, w13, chunked: bool = False,
+                             activation: str = "silu"):
+    """act(n W1^T) * (n W3^T) with n the normed rows given by their two halves; ``chunked``:
     as :class:`ChunkedRows`, for :func:`skinny_into_chain` to read."""
     _check_chain(xg, ssq, w13, "skinny_after_chain_gated")
     M, K = xg.shape
@@ -194,7 +205,8 @@ def skinny_after_chain_gated(xg, ssq, eps: float, w13, chunked: bool = False):
         res = out = torch.empty((M, I), dtype=torch.bfloat16, device=w13.device)
     check(library("gemm_bf16").gfa_skinny_after_chain_bf16(
         ptr(xg.data), ptr(ssq), _i(ssq.shape[0]), ctypes.c_float(eps), ptr(w13), ptr(out), _i(M), _i(I),
-        _i(K), _i(I), _i(3), _i(I), _i(int(chunked)), stream_handle()), "skinny_after_chain_gated")
+        _i(K), _i(I), _i(_gate_mode(activation)), _i(I), _i(int(chunked)), stream_handle()),
+        "skinny_after_chain_gated")
     return res
 
 

@@ -268,18 +268,19 @@ GATE_ACTIVATIONS = K.GATE_ACTIVATIONS
 
 def gated_linear(x: torch.Tensor, w13: torch.Tensor, activation: str = "silu"):
     """[M, I] = act(x W1^T) * (x W3^T), with w13 = rows of W1 then rows of W3
-    (model.py:227).  The products whose epilogue applies the gate know silu; another
-    activation runs the product, then the gate kernel."""
-    if activation != "silu":
-        if isinstance(x, HalfNormed):
-            raise KernelError("a norm in two halves feeds the silu gate's kernels only")
-        return K.gate_mul(linear(x, w13), activation)
+    (model.py:227).  The few-row kernels apply either activation in their epilogue; with more
+    rows only silu has such kernels, and gelu runs the product, then the gate kernel."""
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"gate activation '{activation}': {sorted(GATE_ACTIVATIONS)}")
     if isinstance(x, HalfNormed):
-        return _fast().skinny_after_chain_gated(x.xg, x.ssq, x.eps, w13)
+        return _fast().skinny_after_chain_gated(x.xg, x.ssq, x.eps, w13, activation=activation)
     if x.dtype == torch.float32:
-        return K.silu_mul(K.gemm_f32(x, w13))
+        return K.gate_mul(K.gemm_f32(x, w13), activation)
     if x.shape[0] <= SKINNY_MAX_ROWS:
-        return _fast().skinny_gated(x, w13)
+        return _fast().skinny_gated(x, w13, activation=activation)
+    if activation != "silu":
+        # beyond sixteen rows only silu has kernels with the gate in their epilogue
+        return K.gate_mul(linear(x, w13), activation)
     t = _tiled_for(x.shape[0], w13, gate=True) if w13.shape[0] % 2 == 0 else None
     if t is not None:
         from . import gemm_tiled_bf16 as T
@@ -295,9 +296,9 @@ def gated_into(x, w13: torch.Tensor, w2: torch.Tensor, residual: torch.Tensor, t
     :func:`linear_into` with its arguments and result.  Between two few-row kernels that take
     and leave a norm in halves, the gate's result stays in the order the second one loads it
     in (``gemm_bf16.ChunkedRows``)."""
-    if activation == "silu" and isinstance(x, HalfNormed) \
-            and _chains(x.shape[0], x.dtype, w2, then_norm, takes_halves):
-        h = _fast().skinny_after_chain_gated(x.xg, x.ssq, x.eps, w13, chunked=True)
+    if isinstance(x, HalfNormed) and _chains(x.shape[0], x.dtype, w2, then_norm, takes_halves):
+        h = _fast().skinny_after_chain_gated(x.xg, x.ssq, x.eps, w13, chunked=True,
+                                             activation=activation)
     else:
         h = gated_linear(x, w13, activation)
     return linear_into(h, w2, residual, then_norm, takes_halves)

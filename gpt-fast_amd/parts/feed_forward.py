@@ -29,9 +29,7 @@ class GatedFeedForward(Part):
     # x may be an ops.linear.HalfNormed, from one row on (the least number of rows; with the
     # weights streamed past the caches the matrix-core kernel that takes the halves is as fast
     # at one row as the dot-product kernel that does not, and the norm kernel is saved)
-    @property
-    def takes_prepared(self):
-        return 1 if self.spec.activation == "silu" else False
+    takes_prepared = 1
 
     def step_flops(self, q_lens, starts) -> float:
         return 2.0 * sum(q_lens) * 3 * self.spec.hidden * self.spec.dim

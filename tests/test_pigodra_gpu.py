@@ -75,6 +75,21 @@ def test_gelu_gate_kernel():
                            torch.nn.functional.silu(g[:, :width // 2]) * g[:, width // 2:]) < tol
 
 
+@pytest.mark.parametrize("rows", [1, 3, 8, 16, 17, 40, 100])
+def test_gated_product_with_the_gelu_gate(rows):
+    """Few rows: the gate in the product's epilogue; more: the product, then the gate kernel."""
+    from gpt_fast_amd.ops import linear as L
+    torch.manual_seed(rows)
+    for K_, I in ((96, 136), (104, 52), (256, 320)):
+        x = torch.randn(rows, K_, device=DEV).bfloat16()
+        w13 = (torch.randn(2 * I, K_, device=DEV) * 0.2).bfloat16()
+        gu = x.double().cpu() @ w13.double().cpu().T
+        want = P.gelu_tanh(gu[:, :I]) * gu[:, I:]
+        assert rel_err(L.gated_linear(x, w13, "gelu_tanh"), want) < 1e-2
+        xf, wf = x.float(), w13.float()
+        assert rel_err(L.gated_linear(xf, wf, "gelu_tanh"), want) < 1e-5
+
+
 def test_norm_with_weights_stored_around_zero():
     from gpt_fast_amd.config.spec import NormSpec
     from gpt_fast_amd.parts.base import NORMS, Runtime
