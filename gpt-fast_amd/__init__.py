@@ -1,4 +1,5 @@
-"""An MI355X-native generation library for the Llama 2/3 dense decoder.
+"""An MI355X-native generation library for the Llama 2/3 dense decoder and the Pigodra stack
+(matrix-memory and differential-attention layers).
 
 From a model folder (``config.json`` + safetensors) or seeded random weights to
 generated tokens, through hand-written HIP kernels for gfx950:

@@ -26,6 +26,8 @@ __global__ __launch_bounds__(256) void da_rope_store_kernel(
         const int* __restrict__ tok_pos, const int* __restrict__ table, int table_stride, int H,
         int G, int dim, int vdim, int rot) {
     extern __shared__ float cs[];                          // [rot / 2][2]
+    // blockIdx.y walks the token's elements in groups of 256; each workgroup works out the
+    // token's cos and sin for itself
     const int n = blockIdx.x;
     const int pos = tok_pos[n];
     for (int i = threadIdx.x; i < rot / 2; i += 256)
@@ -36,7 +38,8 @@ __global__ __launch_bounds__(256) void da_rope_store_kernel(
     if (k_pages) page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
     const int off = pos % GFA_PAGE;
     const int q_elems = H * DA_MAPS * dim, k_elems = G * DA_MAPS * dim, v_elems = G * vdim;
-    for (int e = threadIdx.x; e < q_elems + k_elems + v_elems; e += 256) {
+    const int e = blockIdx.y * 256 + threadIdx.x;
+    if (e < q_elems + k_elems + v_elems) {
         if (e < q_elems + k_elems) {
             const bool is_q = e < q_elems;
             const int ee = is_q ? e : e - q_elems;
@@ -73,12 +76,15 @@ extern "C" int gfa_da_rope_store(const void* proj, int row_width, int q_off, int
                                  int rot, int is_bf16, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     const size_t shmem = (size_t)(rot > 0 ? rot : 2) * sizeof(float);
+    const int elems = (H + G) * DA_MAPS * dim + G * vdim;
+    if ((elems + 255) / 256 > 65535) return (int)hipErrorInvalidValue;
+    const dim3 grid(n_tokens, (elems + 255) / 256);
     if (is_bf16)
-        da_rope_store_kernel<bf16_t><<<n_tokens, 256, shmem, stream>>>(
+        da_rope_store_kernel<bf16_t><<<grid, 256, shmem, stream>>>(
             (const bf16_t*)proj, row_width, q_off, k_off, v_off, (bf16_t*)q_out, (bf16_t*)k_pages,
             (bf16_t*)v_pages, freqs, tok_seq, tok_pos, table, table_stride, H, G, dim, vdim, rot);
     else
-        da_rope_store_kernel<float><<<n_tokens, 256, shmem, stream>>>(
+        da_rope_store_kernel<float><<<grid, 256, shmem, stream>>>(
             (const float*)proj, row_width, q_off, k_off, v_off, (float*)q_out, (float*)k_pages,
             (float*)v_pages, freqs, tok_seq, tok_pos, table, table_stride, H, G, dim, vdim, rot);
     return GFA_LAUNCH_RESULT();
