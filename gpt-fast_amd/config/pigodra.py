@@ -172,8 +172,8 @@ def _stack(width: int, n_layers: int, ff: int, kv_heads: int, vocab: int = 32000
         if i % 4 == 3:
             layers.append(PigodraLayer("attention", DifferentialMixer(
                 heads=heads // 2, kv_heads=max(1, kv_heads // 2), dim=128, vdim=256, scale=None,
-                diff=0.3, window=window, keep_first=4, rot_dims=64, rot_base=250000.0,
-                rot_factor=2.0), DenseMlp(ff)))
+                diff=0.2, window=window, keep_first=8, rot_dims=64, rot_base=500000.0,
+                rot_factor=4.0), DenseMlp(ff)))
         else:
             layers.append(PigodraLayer("mlstm", MatrixMemoryMixer(
                 heads=heads, dim=128, vdim=128, gate_cap=15.0), DenseMlp(ff)))

@@ -14,7 +14,7 @@ import zlib
 import torch
 
 
-def _att(heads, kv, dim, vdim, size, first, rot, base=10000.0, factor=None, scale=None, diff=0.3,
+def _att(heads, kv, dim, vdim, size, first, rot, base=10000.0, factor=None, scale=None, diff=0.25,
          ff=None):
     m = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "diff": diff,
          "mask": {"size": size, "keep_first": first},

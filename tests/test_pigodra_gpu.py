@@ -33,6 +33,8 @@ def bf16_close(got, want):
     rows is held to the tolerance and every row to a bound that a wrong key, a lost state or
     a missing term would still break."""
     e = row_errors(got, want)
+    if e.numel() < 20:               # a handful of rows has no bulk: the wide bound alone
+        return float(e.max()) < 0.35
     return float(e.quantile(0.9)) < TOL_BF16 and float(e.max()) < 0.35
 
 
@@ -491,3 +493,60 @@ def test_command_line_entry_point(tmp_path):
                    checkpoint_path=folder, dtype="float32", device=DEV, out=lines.append)
     assert res["result"].tokens[0] == P.greedy_generate(w, cfg, prompt, 8)
     assert any("tokens/sec" in str(l) for l in lines)
+
+
+def test_trace_replay_program(tmp_path):
+    """bin/trace_run as a program on a Pigodra folder: two batches of unequal requests one after
+    the other (the second takes the slots, state and pages the first gave back), logits wanted
+    at some places only, steps in which nothing is wanted, a request that ends in the step that
+    brings its prompt; max-tokens counts the tokens alone."""
+    import json
+    import os
+    import subprocess
+
+    import numpy as np
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = make_folder(tmp_path, "A", seed=19)
+    cfg, w = P.load_folder(folder)
+    V = cfg["vocab"]
+    reqs = {"a": util.random_tokens(V, 150, 1), "b": util.random_tokens(V, 9, 2), "c": util.random_tokens(V, 1, 3),
+            "d": util.random_tokens(V, 200, 4), "e": util.random_tokens(V, 70, 5)}
+    prompt = {"a": 120, "b": 3, "c": 1, "d": 130, "e": 64}
+    steps, where = [], {r: [] for r in reqs}          # request -> (step, row in the file, position)
+    n = 0
+    for ids in (["a", "b", "c"], ["d", "e"]):
+        live, t = list(ids), 0
+        while live:
+            entries, row = [], 0
+            for r in live:
+                lo, hi = (0, prompt[r]) if t == 0 else (prompt[r] + t - 1, prompt[r] + t)
+                want = [i for i in range(hi - lo) if (lo + i) % 3 != 1]
+                entries.append({"id": r, "tokens": reqs[r][lo:hi], "want": want})
+                for i in want:
+                    where[r].append((n, row, lo + i))
+                    row += 1
+            ending = [r for r in live if prompt[r] + t >= len(reqs[r])]
+            steps.append({"step": n, "entries": entries, "end": ending})
+            live = [r for r in live if r not in ending]
+            n += 1
+            t += 1
+    lines = "\n".join(json.dumps(s) for s in steps) + "\n"
+    for dtype in ("float32", "bfloat16"):
+        out = str(tmp_path / dtype)
+        proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                               "--out", out, "--max-tokens", str(200 + 70)],
+                              input=lines, capture_output=True, text=True, timeout=110)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+        for r, toks in reqs.items():
+            want = P.forward(w, cfg, toks)
+            rows, places = [], []
+            for step, row, pos in where[r]:
+                data = np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, V)
+                rows.append(torch.from_numpy(data[row].copy()))
+                places.append(pos)
+            assert close(torch.stack(rows), want[places], dtype, TOL_F32_LONG), (dtype, r)
+        # a step in which nothing is wanted writes no file
+        for s in steps:
+            if not any(e["want"] for e in s["entries"]):
+                assert not os.path.exists(os.path.join(out, f"{s['step']}.f32"))
