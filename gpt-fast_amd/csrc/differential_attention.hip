@@ -1,4 +1,5 @@
-// Differential attention over the paged cache: plain kernels.
+// Differential attention over the paged cache: the rotation and cache write, a plain
+// attention kernel (float32 and any size), and one on the matrix cores (bfloat16).
 //
 // A head holds MAPS = 2 softmax maps over the same values.  Query rows lie head by head as
 // [map 1, map 2], each map `dim` wide; so do key rows per kv head; values are `vdim` wide.

@@ -1,4 +1,6 @@
-// Recurrent mixer with a matrix memory per head (the mLSTM cell): plain kernels.
+// Recurrent mixer with a matrix memory per head (the mLSTM cell): a kernel that goes token by
+// token (single-token steps), one that takes a chunk of tokens at a time (prompts), and the
+// head norm and gate that follow the cell.
 //
 // Per sequence and head the state is S [dk, dv], n [dk] and a running maximum m of the log
 // gates, all float and kept in the cache's state slots:
