@@ -57,6 +57,11 @@ CASES = {
     ]),
     # memory layers only, keys wider than values and the other way round
     "M": _model(64, 97, 1e-5, 0.25, [_mem(2, 64, 16, 10.0), _mem(4, 8, 48, 6.0, ff=40)]),
+    # a width and head sizes that are multiples of two only: no kernel's fast form applies
+    "O": _model(100, 131, 1e-5, 0.8, [
+        _mem(2, 10, 6, 5.0),
+        _att(2, 1, 10, 6, 9, 2, 4, ff=36, factor=3.0),
+    ]),
     # attention layers only, no window (every earlier key) and no rotation
     "T": _model(72, 150, 1e-6, 2.0, [
         _att(3, 3, 16, 24, None, 0, 0, ff=64),

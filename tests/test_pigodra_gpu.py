@@ -107,7 +107,8 @@ def test_norm_with_weights_stored_around_zero():
 
 
 @pytest.mark.parametrize("H,dk,dv,cap", [(2, 16, 32, 8.0), (1, 24, 40, None), (3, 20, 12, 3.0),
-                                         (2, 72, 8, 15.0), (1, 130, 33, 5.0)])
+                                         (2, 72, 8, 15.0), (1, 130, 33, 5.0), (3, 10, 6, 4.0),
+                                         (2, 128, 128, 12.0)])
 @pytest.mark.parametrize("chunked", [False, True])
 def test_memory_cell_kernels_alone(H, dk, dv, cap, chunked):
     """Three sequences of unequal length in one launch, then a second launch that goes on
@@ -243,7 +244,7 @@ def _attention_alone(dtype, H, G, dim, vdim, window, first, rot, lens, starts, b
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
 @pytest.mark.parametrize("H,G,dim,vdim,window,first,rot", [
     (4, 2, 16, 32, 24, 3, 16), (3, 1, 24, 24, 7, 0, 8), (2, 2, 20, 40, 90, 70, 20),
-    (6, 3, 8, 16, 0, 0, 0), (2, 1, 32, 64, 64, 1, 16), (1, 1, 36, 18, 65, 64, 12)])
+    (6, 3, 8, 16, 0, 0, 0), (2, 1, 32, 64, 64, 1, 16), (1, 1, 36, 18, 65, 64, 12), (2, 1, 10, 6, 9, 2, 4)])
 def test_attention_kernels_alone(dtype, tol, H, G, dim, vdim, window, first, rot):
     # prompts from the start, portions at an offset, single tokens far into a sequence
     assert _attention_alone(dtype, H, G, dim, vdim, window, first, rot, [150, 1, 70], [0, 0, 0]) < tol
@@ -314,7 +315,7 @@ def test_a_loud_key_at_the_windows_edge_and_among_the_kept_keys(offset, decode):
 
 
 # --------------------------------------------------------------------------- whole models
-@pytest.mark.parametrize("name", ["A", "B", "M", "T"])
+@pytest.mark.parametrize("name", ["A", "B", "M", "T", "O"])
 @pytest.mark.parametrize("dtype,tol", [("float32", TOL_F32_LONG), ("bfloat16", TOL_BF16)])
 def test_whole_prompt_matches_plain_at_every_position(tmp_path, name, dtype, tol):
     folder = make_folder(tmp_path, name, seed=11)
@@ -331,7 +332,7 @@ def test_whole_prompt_matches_plain_at_every_position(tmp_path, name, dtype, tol
         assert rel_err(_steps(eng, toks[:3], []), want[:3]) < TOL_F32
 
 
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "O"])
 @pytest.mark.parametrize("dtype,tol,same", [("float32", TOL_F32_LONG, 2e-5), ("bfloat16", TOL_BF16, TOL_BF16)])
 def test_portions_and_token_by_token_equal_the_whole_prompt(tmp_path, name, dtype, tol, same):
     folder = make_folder(tmp_path, name, seed=12)
