@@ -149,8 +149,8 @@ extern "C" int gfa_matrix_memory_scan(const float* proj, const float* gate_bias,
 }
 
 // --------------------------------------------------------------------------------------
-// The same cell for runs of many tokens, a chunk of MC_L tokens at a time instead of token by
-// token.  Inside a chunk that starts from (S0, n0, m0), with F_t the running sum of the log
+// The same cell for runs of many tokens, a chunk of MC_L (32 or 64) tokens at a time instead
+// of token by token.  Inside a chunk that starts from (S0, n0, m0), with F_t the running sum of the log
 // forget gates from the chunk's start, g_s = i_s - F_s and M_t = max(m0, max_{s<=t} g_s):
 //     m_t = F_t + M_t
 //     S_t^T q_t = exp(m0 - M_t) S0^T q_t + sum_{s<=t} exp(g_s - M_t) (k_s . q_t) v_s
@@ -158,11 +158,9 @@ extern "C" int gfa_matrix_memory_scan(const float* proj, const float* gate_bias,
 // and the state after the chunk's last token L is
 //     S_L = exp(m0 - M_L) S0 + sum_s exp(g_s - M_L) k_s v_s^T        (n_L likewise)
 // which is the recurrence written out; every exponent is <= 0.  All float.
-// grid (dv / MC_COLS, H, sequences), 256 threads; q, k, v of the chunk, the weighted scores
+// grid (dv / MC_COLS, H, sequences), eight threads per token of a chunk; q, k, v of the chunk, the weighted scores
 // and the workgroup's columns of S are in shared memory.
-#define MC_L 32
 #define MC_COLS 32
-#define MC_PS (MC_L + 1)
 
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float mc_floatx4_t;
 
@@ -171,11 +169,15 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float mc_floatx4_t;
 __host__ __device__ inline int mc_padded(int dk) { return (dk + 15) / 16 * 16; }
 __host__ __device__ inline int mc_row_stride(int dk) { return mc_padded(dk) + 4; }
 
-__global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
+template <int MC_L>
+__global__ __launch_bounds__(MC_L * 8) void matrix_memory_chunk_kernel(
         const float* __restrict__ proj, const float* __restrict__ gate_bias,
         float* __restrict__ state, size_t slot_stride, const int* __restrict__ q_start,
         const int* __restrict__ slots, float* __restrict__ out, MMShape s) {
     extern __shared__ __attribute__((aligned(16))) float mc_lds[];
+    constexpr int NT = MC_L * 8;                 // threads: eight per token of a chunk
+    constexpr int NWV = NT / 64;                 // waves
+    constexpr int MC_PS = MC_L + 1;
     const int KS = mc_row_stride(s.dk);
     const int dkp = mc_padded(s.dk);
     float* Qs = mc_lds;                          // [MC_L][KS]
@@ -199,12 +201,12 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
     float* const mptr = base + (size_t)s.H * s.dk * (s.dv + 1) + h;
     const float ib = gate_bias[h], fb = gate_bias[s.H + h];
 
-    for (int e = tid; e < dkp * MC_COLS; e += 256) {
+    for (int e = tid; e < dkp * MC_COLS; e += NT) {
         const int d = e / MC_COLS, c = e % MC_COLS;
         Ss[e] = (d < s.dk && col0 + c < s.dv) ? S[(size_t)d * s.dv + col0 + c] : 0.f;
     }
-    for (int d = tid; d < dkp; d += 256) ns[d] = d < s.dk ? nvec[d] : 0.f;
-    for (int e = tid; e < 2 * MC_L * KS; e += 256) Qs[e] = 0.f;      // q and k: the filling stays zero
+    for (int d = tid; d < dkp; d += NT) ns[d] = d < s.dk ? nvec[d] : 0.f;
+    for (int e = tid; e < 2 * MC_L * KS; e += NT) Qs[e] = 0.f;      // q and k: the filling stays zero
     float m_prev = *mptr;
 
     // The rows of a chunk come from memory a chunk ahead: they are asked for before the chunk
@@ -221,7 +223,7 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
         const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int e = tid + 256 * i, t = e / kq4, d4 = e - t * kq4;
+            const int e = tid + NT * i, t = e / kq4, d4 = e - t * kq4;
             rq[i] = rk[i] = zero;
             if (t < Lc) {
                 const float* row = proj + (size_t)(c0 + t) * s.row_width + h * s.dk + d4 * 4;
@@ -250,7 +252,7 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
         if (vec) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int e = tid + 256 * i, t = e / kq4, d4 = e - t * kq4;
+                const int e = tid + NT * i, t = e / kq4, d4 = e - t * kq4;
                 if (t < MC_L) {
                     float4 x = rq[i];
                     x.x *= s.q_scale; x.y *= s.q_scale; x.z *= s.q_scale; x.w *= s.q_scale;
@@ -264,14 +266,14 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
             if (c0 + MC_L < t1) fetch(c0 + MC_L);
         } else {
             // q (scaled), k, v of the chunk; rows beyond its end and columns beyond dk are zero
-            for (int e = tid; e < MC_L * KS; e += 256) {
+            for (int e = tid; e < MC_L * KS; e += NT) {
                 const int t = e / KS, d = e - t * KS;
                 const bool ok = t < Lc && d < s.dk;
                 const float* row = proj + (size_t)(c0 + t) * s.row_width;
                 Qs[e] = ok ? row[s.q_off + h * s.dk + d] * s.q_scale : 0.f;
                 Ks[e] = ok ? row[s.k_off + h * s.dk + d] : 0.f;
             }
-            for (int e = tid; e < MC_L * MC_COLS; e += 256) {
+            for (int e = tid; e < MC_L * MC_COLS; e += NT) {
                 const int t = e / MC_COLS, c = e % MC_COLS;
                 Vs[e] = (t < Lc && col0 + c < s.dv)
                     ? proj[(size_t)(c0 + t) * s.row_width + s.v_off + h * s.dv + col0 + c] : 0.f;
@@ -317,16 +319,17 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
         // a 16 x 16 tile of the result per wave and loop.
         const int li = lane & 15, lg = lane >> 4;
         // scores of the chunk, weighted: P[t][s] = (q_t . k_s) exp(g_s - M_t) for s <= t
-        {
-            const int ti = wave >> 1, si = wave & 1;
+        // (the 16 x 16 tiles on and below the diagonal, handed out over the waves)
+        for (int idx = wave; idx < (MC_L / 16) * (MC_L / 16 + 1) / 2; idx += NWV) {
+            int ti = 0;
+            while ((ti + 1) * (ti + 2) / 2 <= idx) ++ti;
+            const int si = idx - ti * (ti + 1) / 2;
             mc_floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
-            if (si <= ti) {                       // the tile above the diagonal is all zero
-                const float* qa = Qs + (ti * 16 + li) * KS + lg;
-                const float* kb = Ks + (si * 16 + li) * KS + lg;
+            const float* qa = Qs + (ti * 16 + li) * KS + lg;
+            const float* kb = Ks + (si * 16 + li) * KS + lg;
 #pragma unroll 4
-                for (int d0 = 0; d0 < dkp; d0 += 4)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[d0], kb[d0], acc, 0, 0, 0);
-            }
+            for (int d0 = 0; d0 < dkp; d0 += 4)
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[d0], kb[d0], acc, 0, 0, 0);
             const int ss = si * 16 + li;
             const float g = gs[ss];
 #pragma unroll
@@ -384,7 +387,7 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
         // rows of S by 16 columns in turn
         {
             const float decay = expf(m_prev - Ms[Lc - 1]);
-            for (int tile = wave; tile < (dkp / 16) * 2; tile += 4) {
+            for (int tile = wave; tile < (dkp / 16) * 2; tile += NWV) {
                 const int di = tile >> 1, ci = tile & 1;
                 float* sc = Ss + (di * 16 + lg * 4) * MC_COLS + ci * 16 + li;
                 mc_floatx4_t acc;
@@ -399,7 +402,7 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
 #pragma unroll
                 for (int r = 0; r < 4; ++r) sc[r * MC_COLS] = acc[r];
             }
-            for (int d = tid; d < s.dk; d += 256) {
+            for (int d = tid; d < s.dk; d += NT) {
                 float a = decay * ns[d];
                 for (int ss = 0; ss < Lc; ++ss) a = fmaf(ws[ss], Ks[ss * KS + d], a);
                 ns[d] = a;
@@ -408,34 +411,73 @@ __global__ __launch_bounds__(256) void matrix_memory_chunk_kernel(
         }
     }
     __syncthreads();
-    for (int e = tid; e < s.dk * MC_COLS; e += 256) {
+    for (int e = tid; e < s.dk * MC_COLS; e += NT) {
         const int d = e / MC_COLS, c = e % MC_COLS;
         if (col0 + c < s.dv) S[(size_t)d * s.dv + col0 + c] = Ss[e];
     }
     if (blockIdx.x == 0) {
-        for (int d = tid; d < s.dk; d += 256) nvec[d] = ns[d];
+        for (int d = tid; d < s.dk; d += NT) nvec[d] = ns[d];
         if (tid == 0) *mptr = m_prev;
     }
 }
 
-extern "C" int gfa_matrix_memory_chunk_lds(int dk) {
+static int mc_lds_bytes(int dk, int L) {
     const int dkp = mc_padded(dk);
-    return (int)sizeof(float) * (2 * MC_L * mc_row_stride(dk) + MC_L * MC_COLS + MC_L * MC_PS
-                                 + dkp * MC_COLS + dkp + 5 * MC_L);
+    return (int)sizeof(float) * (2 * L * mc_row_stride(dk) + L * MC_COLS + L * (L + 1)
+                                 + dkp * MC_COLS + dkp + 5 * L);
 }
 
+static int mc_lds_limit() {
+    static int limit = -1;
+    if (limit < 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess)
+            v = 64 * 1024;
+        limit = v;
+    }
+    return limit;
+}
+
+// 1 if chunks of 64 tokens fit a workgroup's shared memory on this device for this key size
+extern "C" int gfa_matrix_memory_long_chunks(int dk) {
+    return dk <= 128 && mc_lds_bytes(dk, 64) <= mc_lds_limit() ? 1 : 0;
+}
+
+// Chunks of 64 tokens (512 threads) where the device lets a workgroup have the shared memory
+// for them (109 KB at dk = 128), else chunks of 32 (256 threads, at most 60 KB): a longer
+// chunk spreads the chain of barriers, the gates' scans and the state's products over twice
+// the tokens.
 extern "C" int gfa_matrix_memory_chunks(const float* proj, const float* gate_bias, float* state,
                                         size_t slot_stride, const int* q_start, const int* slots,
                                         float* out, int n_seqs, int H, int dk, int dv, int row_width,
                                         int q_off, int k_off, int v_off, int i_off, int f_off,
-                                        float q_scale, float cap, float den_eps, hipStream_t stream) {
+                                        float q_scale, float cap, float den_eps, int chunk,
+                                        hipStream_t stream) {
     if (n_seqs <= 0) return 0;
-    const int shmem = gfa_matrix_memory_chunk_lds(dk);
-    if (dk > 128 || shmem > 64 * 1024 || H > 65535 || n_seqs > 65535) return (int)hipErrorInvalidValue;
+    if (dk > 128 || H > 65535 || n_seqs > 65535 || (chunk != 0 && chunk != 32 && chunk != 64))
+        return (int)hipErrorInvalidValue;
+    const int lds_limit = mc_lds_limit();
     MMShape s{H, dk, dv, row_width, q_off, k_off, v_off, i_off, f_off, q_scale, cap, den_eps};
     dim3 grid((dv + MC_COLS - 1) / MC_COLS, H, n_seqs);
-    matrix_memory_chunk_kernel<<<grid, 256, shmem, stream>>>(proj, gate_bias, state, slot_stride,
-                                                             q_start, slots, out, s);
+    const int big = mc_lds_bytes(dk, 64);
+    if (chunk == 64 && big > lds_limit) return (int)hipErrorInvalidValue;
+    if (chunk != 32 && big <= lds_limit) {
+        static bool allowed = false;
+        if (!allowed) {
+            const hipError_t e = hipFuncSetAttribute((const void*)matrix_memory_chunk_kernel<64>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return (int)e;
+            allowed = true;
+        }
+        matrix_memory_chunk_kernel<64><<<grid, 512, big, stream>>>(proj, gate_bias, state, slot_stride,
+                                                                  q_start, slots, out, s);
+        return GFA_LAUNCH_RESULT();
+    }
+    const int small = mc_lds_bytes(dk, 32);
+    if (small > 64 * 1024) return (int)hipErrorInvalidValue;
+    matrix_memory_chunk_kernel<32><<<grid, 256, small, stream>>>(proj, gate_bias, state, slot_stride,
+                                                                q_start, slots, out, s);
     return GFA_LAUNCH_RESULT();
 }
 

@@ -57,10 +57,11 @@ def cell(proj, layout, gate_bias, state, q_start, slots, n_seqs, max_q_len, n_he
 def scan(proj: torch.Tensor, layout: RowLayout, gate_bias: torch.Tensor, state: torch.Tensor,
          q_start: torch.Tensor, slots: torch.Tensor, n_seqs: int, n_heads: int, key_dim: int,
          value_dim: int, q_scale: float, gate_cap: float, den_eps: float,
-         chunked: bool = False) -> torch.Tensor:
+         chunked: bool = False, chunk: int = 0) -> torch.Tensor:
     """The cell over every sequence's new tokens in order; ``state`` [slots, state_size] is
     read and left updated.  proj float32 [N, layout.width]; returns o float32 [N, H, dv].
-    ``chunked``: the kernel that takes 32 tokens at a time (key_dim up to 128)."""
+    ``chunked``: the kernel that takes ``chunk`` = 32 or 64 tokens at a time (key_dim up to
+    128; 0: 64 where the device's shared memory holds them, else 32)."""
     require_device(proj, gate_bias, state, q_start, slots)
     require_contiguous(proj=proj, gate_bias=gate_bias, state=state, q_start=q_start, slots=slots)
     for name, t in (("proj", proj), ("gate_bias", gate_bias), ("state", state)):
@@ -86,14 +87,22 @@ def scan(proj: torch.Tensor, layout: RowLayout, gate_bias: torch.Tensor, state: 
     out = torch.empty((proj.shape[0], n_heads, value_dim), dtype=torch.float32, device=proj.device)
     if chunked and key_dim > CHUNK_MAX_KEY_DIM:
         raise KernelError(f"matrix memory: the chunked kernel takes key_dim up to {CHUNK_MAX_KEY_DIM}")
-    entry = (library("matrix_memory").gfa_matrix_memory_chunks if chunked
-             else library("matrix_memory").gfa_matrix_memory_scan)
-    check(entry(
-        ptr(proj), ptr(gate_bias), ptr(state), _sz(state.stride(0)), ptr(q_start), ptr(slots),
-        ptr(out), _i(n_seqs), _i(n_heads), _i(key_dim), _i(value_dim), _i(layout.width),
-        _i(layout.q), _i(layout.k), _i(layout.v), _i(layout.i), _i(layout.f), _f(q_scale),
-        _f(gate_cap or 0.0), _f(den_eps), stream_handle()), "matrix_memory_scan")
+    args = (ptr(proj), ptr(gate_bias), ptr(state), _sz(state.stride(0)), ptr(q_start), ptr(slots),
+            ptr(out), _i(n_seqs), _i(n_heads), _i(key_dim), _i(value_dim), _i(layout.width),
+            _i(layout.q), _i(layout.k), _i(layout.v), _i(layout.i), _i(layout.f), _f(q_scale),
+            _f(gate_cap or 0.0), _f(den_eps))
+    if chunked:
+        check(library("matrix_memory").gfa_matrix_memory_chunks(*args, _i(chunk), stream_handle()),
+              "matrix_memory_chunks")
+    else:
+        check(library("matrix_memory").gfa_matrix_memory_scan(*args, stream_handle()),
+              "matrix_memory_scan")
     return out
+
+
+def long_chunks_available(key_dim: int) -> bool:
+    """Chunks of 64 tokens fit a workgroup's shared memory on the current device."""
+    return bool(library("matrix_memory").gfa_matrix_memory_long_chunks(_i(key_dim)))
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, proj: torch.Tensor, layout: RowLayout,
