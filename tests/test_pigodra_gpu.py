@@ -388,6 +388,45 @@ def test_unequal_batches_equal_each_request_alone(tmp_path, name, dtype, same):
     assert close(torch.cat(got[2]), want, dtype, TOL_F32_LONG)
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_step_that_mixes_single_tokens_a_portion_and_a_new_prompt(tmp_path, name, dtype):
+    """Three sequences go on by one token, one by a portion of 40 tokens at position 70 and one
+    starts with 130 tokens, all in one step (the generation loop makes no such step; the step
+    function takes it)."""
+    import gpt_fast_amd as gfa
+    folder = make_folder(tmp_path, name, seed=21)
+    cfg, w = P.load_folder(folder)
+    seqs, before, mixed = util.mixed_step_case(cfg["vocab"])
+    eng = _engine(folder, dtype, max_tokens=64 * 16, max_sequences=5)
+    slots = {r: eng.start_sequence() for r in seqs}
+    got = {r: [] for r in seqs}
+    order = ["d0", "d1", "d2", "c"]
+    logits = eng.step([gfa.Entry(slots[r], seqs[r][:before[r]], want=list(range(before[r]))) for r in order]).cpu()
+    at = 0
+    for r in order:
+        got[r].append(logits[at:at + before[r]])
+        at += before[r]
+    order = ["d0", "c", "d1", "p", "d2"]
+    fed = {r: before.get(r, 0) for r in order}
+    logits = eng.step([gfa.Entry(slots[r], seqs[r][fed[r]:fed[r] + mixed[r]], want=list(range(mixed[r])))
+                       for r in order]).cpu()
+    at = 0
+    for r in order:
+        got[r].append(logits[at:at + mixed[r]])
+        at += mixed[r]
+        fed[r] += mixed[r]
+    for r in ("c", "p"):
+        while fed[r] < len(seqs[r]):
+            got[r].append(eng.step([gfa.Entry(slots[r], [seqs[r][fed[r]]], want=[0])]).cpu())
+            fed[r] += 1
+    for r, toks in seqs.items():
+        assert close(torch.cat(got[r]), P.forward(w, cfg, toks), dtype, TOL_F32_LONG), r
+        eng.end_sequence(slots[r])
+    eng.cache.check()
+    assert eng.cache.slots.held == 0
+
+
 def test_slots_and_pages_that_come_back_start_clean(tmp_path):
     """A cache of few pages and two slots: requests follow one another in the same slots and
     pages, long decoding gives the window's pages back, and every request equals the plain
