@@ -15,17 +15,19 @@
 #define DA_MAPS 2
 
 // --------------------------------------------------------------------------------------
-// Rotation of q and k and the cache write.  proj [N, row_width] holds per token
-// q [H][2][dim] at q_off, k [G][2][dim] at k_off, v [G][vdim] at v_off.  Pairs (2i, 2i+1) of
-// the first `rot` elements of every map are rotated by pos * freqs[i], angle, cos and sin in
-// float; the rest passes through.  q goes to q_out [N, H, 2, dim].
+// Rotation of q and k and the cache write.  proj [N, row_width], float (the projection's
+// accumulators, unrounded), holds per token q [H][2][dim] at q_off, k [G][2][dim] at k_off,
+// v [G][vdim] at v_off and, if gate_out is given, one gate number per head at g_off.  Pairs
+// (2i, 2i+1) of the first `rot` elements of every map are rotated by pos * freqs[i], angle,
+// cos and sin in float; the rest passes through.  q goes to q_out [N, H, 2, dim], k and v
+// into the pages, each rounded once to T; the gates are copied to gate_out [N, H], float.
 template <typename T>
 __global__ __launch_bounds__(256) void da_rope_store_kernel(
-        const T* __restrict__ proj, int row_width, int q_off, int k_off, int v_off,
+        const float* __restrict__ proj, int row_width, int q_off, int k_off, int v_off, int g_off,
         T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
-        const float* __restrict__ freqs, const int* __restrict__ tok_seq,
-        const int* __restrict__ tok_pos, const int* __restrict__ table, int table_stride, int H,
-        int G, int dim, int vdim, int rot) {
+        float* __restrict__ gate_out, const float* __restrict__ freqs,
+        const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+        const int* __restrict__ table, int table_stride, int H, int G, int dim, int vdim, int rot) {
     extern __shared__ float cs[];                          // [rot / 2][2]
     // blockIdx.y walks the token's elements in groups of 256; each workgroup works out the
     // token's cos and sin for itself
@@ -34,60 +36,67 @@ __global__ __launch_bounds__(256) void da_rope_store_kernel(
     for (int i = threadIdx.x; i < rot / 2; i += 256)
         sincosf((float)pos * freqs[i], &cs[2 * i + 1], &cs[2 * i]);
     __syncthreads();
-    const T* row = proj + (size_t)n * row_width;
+    const float* row = proj + (size_t)n * row_width;
     int page = 0;
     if (k_pages) page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
     const int off = pos % GFA_PAGE;
     const int q_elems = H * DA_MAPS * dim, k_elems = G * DA_MAPS * dim, v_elems = G * vdim;
     const int e = blockIdx.y * 256 + threadIdx.x;
-    if (e < q_elems + k_elems + v_elems) {
-        if (e < q_elems + k_elems) {
-            const bool is_q = e < q_elems;
-            const int ee = is_q ? e : e - q_elems;
-            const int mh = ee / dim, d = ee - mh * dim;    // mh = head * 2 + map
-            const T* src = row + (is_q ? q_off : k_off) + (size_t)mh * dim;
-            float val;
-            if (d < rot) {
-                const int i = d >> 1;
-                const float u = load_as_float(src + 2 * i), w = load_as_float(src + 2 * i + 1);
-                const float c = cs[2 * i], s = cs[2 * i + 1];
-                val = (d & 1) ? w * c + u * s : u * c - w * s;
-            } else {
-                val = load_as_float(src + d);
-            }
-            if (is_q) {
-                store_from_float(q_out + (size_t)n * q_elems + ee, val);
-            } else if (k_pages) {
-                const int g = mh / DA_MAPS, map = mh % DA_MAPS;
-                T* dst = k_pages + cache_region(page, g, G, DA_MAPS * dim) + (size_t)map * GFA_PAGE * dim;
-                store_from_float(dst + key_offset(off, d, dim), val);
-            }
-        } else if (v_pages) {
+    if (e < q_elems + k_elems) {
+        const bool is_q = e < q_elems;
+        const int ee = is_q ? e : e - q_elems;
+        const int mh = ee / dim, d = ee - mh * dim;    // mh = head * 2 + map
+        const float* src = row + (is_q ? q_off : k_off) + (size_t)mh * dim;
+        float val;
+        if (d < rot) {
+            const int i = d >> 1;
+            const float u = src[2 * i], w = src[2 * i + 1];
+            const float c = cs[2 * i], s = cs[2 * i + 1];
+            val = (d & 1) ? w * c + u * s : u * c - w * s;
+        } else {
+            val = src[d];
+        }
+        if (is_q) {
+            store_from_float(q_out + (size_t)n * q_elems + ee, val);
+        } else if (k_pages) {
+            const int g = mh / DA_MAPS, map = mh % DA_MAPS;
+            T* dst = k_pages + cache_region(page, g, G, DA_MAPS * dim) + (size_t)map * GFA_PAGE * dim;
+            store_from_float(dst + key_offset(off, d, dim), val);
+        }
+    } else if (e < q_elems + k_elems + v_elems) {
+        if (v_pages) {
             const int ev = e - q_elems - k_elems;
             const int g = ev / vdim, d = ev - g * vdim;
-            v_pages[cache_region(page, g, G, vdim) + value_offset(d, off, vdim)] = row[v_off + ev];
+            store_from_float(v_pages + cache_region(page, g, G, vdim) + value_offset(d, off, vdim),
+                             row[v_off + ev]);
         }
+    } else if (gate_out && e < q_elems + k_elems + v_elems + H) {
+        const int h = e - q_elems - k_elems - v_elems;
+        gate_out[(size_t)n * H + h] = row[g_off + h];
     }
 }
 
-extern "C" int gfa_da_rope_store(const void* proj, int row_width, int q_off, int k_off, int v_off,
-                                 void* q_out, void* k_pages, void* v_pages, const float* freqs,
-                                 const int* tok_seq, const int* tok_pos, const int* table,
-                                 int table_stride, int n_tokens, int H, int G, int dim, int vdim,
-                                 int rot, int is_bf16, hipStream_t stream) {
+extern "C" int gfa_da_rope_store(const float* proj, int row_width, int q_off, int k_off, int v_off,
+                                 int g_off, void* q_out, void* k_pages, void* v_pages,
+                                 float* gate_out, const float* freqs, const int* tok_seq,
+                                 const int* tok_pos, const int* table, int table_stride,
+                                 int n_tokens, int H, int G, int dim, int vdim, int rot,
+                                 int out_bf16, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     const size_t shmem = (size_t)(rot > 0 ? rot : 2) * sizeof(float);
-    const int elems = (H + G) * DA_MAPS * dim + G * vdim;
+    const int elems = (H + G) * DA_MAPS * dim + G * vdim + H;
     if ((elems + 255) / 256 > 65535) return (int)hipErrorInvalidValue;
     const dim3 grid(n_tokens, (elems + 255) / 256);
-    if (is_bf16)
+    if (out_bf16)
         da_rope_store_kernel<bf16_t><<<grid, 256, shmem, stream>>>(
-            (const bf16_t*)proj, row_width, q_off, k_off, v_off, (bf16_t*)q_out, (bf16_t*)k_pages,
-            (bf16_t*)v_pages, freqs, tok_seq, tok_pos, table, table_stride, H, G, dim, vdim, rot);
+            proj, row_width, q_off, k_off, v_off, g_off, (bf16_t*)q_out, (bf16_t*)k_pages,
+            (bf16_t*)v_pages, gate_out, freqs, tok_seq, tok_pos, table, table_stride, H, G, dim,
+            vdim, rot);
     else
         da_rope_store_kernel<float><<<grid, 256, shmem, stream>>>(
-            (const float*)proj, row_width, q_off, k_off, v_off, (float*)q_out, (float*)k_pages,
-            (float*)v_pages, freqs, tok_seq, tok_pos, table, table_stride, H, G, dim, vdim, rot);
+            proj, row_width, q_off, k_off, v_off, g_off, (float*)q_out, (float*)k_pages,
+            (float*)v_pages, gate_out, freqs, tok_seq, tok_pos, table, table_stride, H, G, dim,
+            vdim, rot);
     return GFA_LAUNCH_RESULT();
 }
 
@@ -101,7 +110,7 @@ extern "C" int gfa_da_rope_store(const void* proj, int row_width, int q_off, int
 template <typename T>
 __global__ __launch_bounds__(DA_THREADS) void da_attention_generic_kernel(
         const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
-        const T* __restrict__ gate, int gate_stride, const int* __restrict__ tok_seq,
+        const float* __restrict__ gate, int gate_stride, const int* __restrict__ tok_seq,
         const int* __restrict__ tok_pos, const int* __restrict__ table, int table_stride,
         T* __restrict__ out, int H, int G, int dim, int vdim, float scale, int window,
         int keep_first, float lam, float eps, float out_scale) {
@@ -184,7 +193,7 @@ __global__ __launch_bounds__(DA_THREADS) void da_attention_generic_kernel(
     }
     ss = block_sum(ss, scratch);
     float f = rsqrtf(ss / (float)vdim + eps) * out_scale;
-    if (gate) f *= 1.f / (1.f + expf(-load_as_float(gate + (size_t)n * gate_stride + h)));
+    if (gate) f *= 1.f / (1.f + expf(-gate[(size_t)n * gate_stride + h]));
     T* orow = out + ((size_t)n * H + h) * vdim;
 #pragma unroll
     for (int i = 0; i < DA_MAX_PER_THREAD; ++i) {
@@ -194,7 +203,7 @@ __global__ __launch_bounds__(DA_THREADS) void da_attention_generic_kernel(
 }
 
 extern "C" int gfa_da_attention_generic(const void* q, const void* k_pages, const void* v_pages,
-                                        const void* gate, int gate_stride, const int* tok_seq,
+                                        const float* gate, int gate_stride, const int* tok_seq,
                                         const int* tok_pos, const int* table, int table_stride,
                                         void* out, int n_tokens, int H, int G, int dim, int vdim,
                                         float scale, int window, int keep_first, float lam,
@@ -206,12 +215,12 @@ extern "C" int gfa_da_attention_generic(const void* q, const void* k_pages, cons
     const size_t shmem = (size_t)(DA_MAPS * dim + DA_MAPS * DA_THREADS + 16) * sizeof(float);
     if (is_bf16)
         da_attention_generic_kernel<bf16_t><<<grid, DA_THREADS, shmem, stream>>>(
-            (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (const bf16_t*)gate,
+            (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, gate,
             gate_stride, tok_seq, tok_pos, table, table_stride, (bf16_t*)out, H, G, dim, vdim,
             scale, window, keep_first, lam, eps, out_scale);
     else
         da_attention_generic_kernel<float><<<grid, DA_THREADS, shmem, stream>>>(
-            (const float*)q, (const float*)k_pages, (const float*)v_pages, (const float*)gate,
+            (const float*)q, (const float*)k_pages, (const float*)v_pages, gate,
             gate_stride, tok_seq, tok_pos, table, table_stride, (float*)out, H, G, dim, vdim,
             scale, window, keep_first, lam, eps, out_scale);
     return GFA_LAUNCH_RESULT();
@@ -256,7 +265,7 @@ __device__ __forceinline__ float da_sum_lane_groups(float v) {
 template <int DK, int DVT, bool SPLIT>
 __global__ __launch_bounds__(SPLIT ? 512 : 256) void da_attention_mfma_kernel(
         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
-        const bf16_t* __restrict__ v_pages, const bf16_t* __restrict__ gate, int gate_stride,
+        const bf16_t* __restrict__ v_pages, const float* __restrict__ gate, int gate_stride,
         const int* __restrict__ q_start, const int* __restrict__ start_pos,
         const int* __restrict__ table, int table_stride, bf16_t* __restrict__ out, int H, int G,
         int dim, int vdim, float scale_log2, int window, int keep_first, float lam, float eps,
@@ -444,7 +453,7 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void da_attention_mfma_kernel(
             }
     ss = da_sum_lane_groups(ss);
     float f = rsqrtf(ss / (float)vdim + eps) * out_scale;
-    if (gate) f *= 1.f / (1.f + expf(-bf16_to_float(gate[(size_t)(q0 + tok) * gate_stride + head])));
+    if (gate) f *= 1.f / (1.f + expf(-gate[(size_t)(q0 + tok) * gate_stride + head]));
     if (!row_ok) return;
     bf16_t* orow = out + ((size_t)(q0 + tok) * H + head) * vdim;
 #pragma unroll
@@ -460,7 +469,7 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void da_attention_mfma_kernel(
 // rows_max: the most rows (tokens times heads of a group) any sequence of the step brings.
 // split_waves > 0: one token per sequence, that many waves share a tile's blocks.
 extern "C" int gfa_da_attention_mfma(const void* q, const void* k_pages, const void* v_pages,
-                                     const void* gate, int gate_stride, const int* q_start,
+                                     const float* gate, int gate_stride, const int* q_start,
                                      const int* start_pos, const int* table, int table_stride,
                                      void* out, int n_seqs, int rows_max, int H, int G, int dim,
                                      int vdim, float scale, int window, int keep_first, float lam,
@@ -478,7 +487,7 @@ extern "C" int gfa_da_attention_mfma(const void* q, const void* k_pages, const v
     const size_t shmem = split_waves > 0 ? (size_t)split_waves * (64 + DA_MAPS * vdim * Rg) * sizeof(float) : 0;
     if (shmem > 64 * 1024) return (int)hipErrorInvalidValue;
 #define DA_LAUNCH(K_, V_, S_) da_attention_mfma_kernel<K_, V_, S_><<<grid, threads, shmem, stream>>>( \
-        (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (const bf16_t*)gate, \
+        (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, gate, \
         gate_stride, q_start, start_pos, table, table_stride, (bf16_t*)out, H, G, dim, vdim, \
         scale_log2, window, keep_first, lam, eps, out_scale)
 #define DA_PICK_V(K_, S_) do { if (dvt == 4) DA_LAUNCH(K_, 4, S_); else if (dvt == 8) DA_LAUNCH(K_, 8, S_); \

@@ -39,17 +39,23 @@ def _check_maps(n, tok_seq, tok_pos, table):
         raise KernelError("token maps are shorter than the batch")
 
 
-def rope_store(proj, q_off, k_off, v_off, freqs, tok_seq, tok_pos, table, k_pages, v_pages,
-               n_heads, n_kv_heads, dim, vdim, rotary_dim):
+def rope_store(proj, q_off, k_off, v_off, g_off, freqs, tok_seq, tok_pos, table, k_pages, v_pages,
+               n_heads, n_kv_heads, dim, vdim, rotary_dim, out_dtype, with_gate=True):
     """Rotate the first ``rotary_dim`` elements (pairs 2i, 2i+1) of every map of q and k of
-    proj [N, width] by position; q to a new [N, H, 2, dim]; k and v into the pages (skipped
-    if they are None)."""
+    proj (float32 [N, width], the projection's unrounded sums) by position; q to a new
+    [N, H, 2, dim] of ``out_dtype``; k and v into the pages of that type (skipped if they are
+    None); the heads' gate numbers at ``g_off`` to a new float32 [N, H] (None without a gate).
+    Returns (q, gate)."""
     require_device(proj, freqs, tok_seq, tok_pos, table, k_pages, v_pages)
     require_contiguous(proj=proj, freqs=freqs, tok_seq=tok_seq, tok_pos=tok_pos, table=table)
+    if proj.dtype != torch.float32 or proj.dim() != 2:
+        raise KernelError("rope_store: the projection's rows must be float32 [N, width]")
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise KernelError(f"rope_store: output type {out_dtype}")
     n, width = proj.shape
     if (q_off + n_heads * MAPS * dim > width or k_off + n_kv_heads * MAPS * dim > width
-            or v_off + n_kv_heads * vdim > width):
-        raise KernelError("rope_store: q, k, v do not fit the rows")
+            or v_off + n_kv_heads * vdim > width or (with_gate and g_off + n_heads > width)):
+        raise KernelError("rope_store: q, k, v and the gates do not fit the rows")
     if rotary_dim % 2 or not 0 <= rotary_dim <= dim:
         raise KernelError(f"rope_store: rotary_dim {rotary_dim} must be even and at most {dim}")
     if rotary_dim and (freqs is None or freqs.dtype != torch.float32 or freqs.numel() != rotary_dim // 2):
@@ -57,19 +63,20 @@ def rope_store(proj, q_off, k_off, v_off, freqs, tok_seq, tok_pos, table, k_page
     _check_maps(n, tok_seq, tok_pos, table)
     if (k_pages is None) != (v_pages is None):
         raise KernelError("rope_store: give both k_pages and v_pages, or neither")
-    _check_pages(k_pages, v_pages, n_kv_heads, dim, vdim, proj.dtype)
-    q_out = torch.empty((n, n_heads, MAPS, dim), dtype=proj.dtype, device=proj.device)
+    _check_pages(k_pages, v_pages, n_kv_heads, dim, vdim, out_dtype)
+    q_out = torch.empty((n, n_heads, MAPS, dim), dtype=out_dtype, device=proj.device)
+    gate = torch.empty((n, n_heads), dtype=torch.float32, device=proj.device) if with_gate else None
     check(library("differential_attention").gfa_da_rope_store(
-        ptr(proj), _i(width), _i(q_off), _i(k_off), _i(v_off), ptr(q_out), ptr(k_pages),
-        ptr(v_pages), ptr(freqs), ptr(tok_seq), ptr(tok_pos), ptr(table), _i(table.shape[1]),
-        _i(n), _i(n_heads), _i(n_kv_heads), _i(dim), _i(vdim), _i(rotary_dim), _i(_is_bf16(proj)),
-        stream_handle()), "da_rope_store")
-    return q_out
+        ptr(proj), _i(width), _i(q_off), _i(k_off), _i(v_off), _i(g_off), ptr(q_out), ptr(k_pages),
+        ptr(v_pages), ptr(gate), ptr(freqs), ptr(tok_seq), ptr(tok_pos), ptr(table),
+        _i(table.shape[1]), _i(n), _i(n_heads), _i(n_kv_heads), _i(dim), _i(vdim), _i(rotary_dim),
+        _i(int(out_dtype == torch.bfloat16)), stream_handle()), "da_rope_store")
+    return q_out, gate
 
 
 def attention_generic(q, k_pages, v_pages, gate, tok_seq, tok_pos, table, scale, window,
                       keep_first, lam, eps, out_scale):
-    """q [N, H, 2, dim]; gate None or a view [N, H] (unit stride along H) of the heads' gate
+    """q [N, H, 2, dim]; gate None or float32 [N, H] (unit stride along H), the heads' gate
     pre-activations.  Returns [N, H * vdim]."""
     require_device(q, k_pages, v_pages, gate, tok_seq, tok_pos, table)
     require_contiguous(q=q, tok_seq=tok_seq, tok_pos=tok_pos, table=table)
@@ -83,8 +90,8 @@ def attention_generic(q, k_pages, v_pages, gate, tok_seq, tok_pos, table, scale,
     _check_maps(n, tok_seq, tok_pos, table)
     gate_stride = 0
     if gate is not None:
-        if gate.shape != (n, H) or gate.dtype != q.dtype or (H > 1 and gate.stride(1) != 1):
-            raise KernelError("differential attention: gate must be [N, H] of q's type")
+        if gate.shape != (n, H) or gate.dtype != torch.float32 or (H > 1 and gate.stride(1) != 1):
+            raise KernelError("differential attention: gate must be float32 [N, H]")
         gate_stride = gate.stride(0)
     out = torch.empty((n, H * vdim), dtype=q.dtype, device=q.device)
     check(library("differential_attention").gfa_da_attention_generic(
@@ -138,8 +145,8 @@ def attention_mfma(q, k_pages, v_pages, gate, q_start, start_pos, table, n_seqs,
         raise KernelError("differential attention: the step's description is shorter than the batch")
     gate_stride = 0
     if gate is not None:
-        if gate.shape != (n, H) or gate.dtype != q.dtype or (H > 1 and gate.stride(1) != 1):
-            raise KernelError("differential attention: gate must be [N, H] of q's type")
+        if gate.shape != (n, H) or gate.dtype != torch.float32 or (H > 1 and gate.stride(1) != 1):
+            raise KernelError("differential attention: gate must be float32 [N, H]")
         gate_stride = gate.stride(0)
     waves = 0
     if single_tokens:

@@ -19,8 +19,9 @@ class DifferentialAttention(Part):
     on their own; the head's result is ``a1 - lam a2`` with
     ``lam = exp(lq1 . lk1) - exp(lq2 . lk2) + lam_init``, divided by its root mean square
     over the value size, times ``1 - lam_init``, times sigmoid of one gate number per head,
-    then ``wo``.  The projections of q, k, v and the gate are one matrix ``w_in``.  Scores,
-    softmax, sums, the combination and the norm are float32."""
+    then ``wo``.  The projections of q, k, v and the gate are one matrix ``w_in`` whose product
+    keeps its float32 sums until the rotation has been applied.  Scores, softmax, sums, the
+    combination, the norm and the gate are float32."""
 
     libraries = ("differential_attention",)
     defers_sum = True              # ``residual`` may be a parts.base.ResidualStream
@@ -92,14 +93,15 @@ class DifferentialAttention(Part):
 
     def forward(self, x, batch, entry, residual):
         s = self.spec
-        proj = L.linear(x, self.w_in)
+        # the projection keeps its float32 sums: q and k are rounded once, after the rotation
+        proj = L.linear(x, self.w_in, out_dtype=torch.float32)
         write = entry is not None and entry.writes
         table = batch.table(entry.group_id)
-        q = DA.rope_store(proj, self.q_off, self.k_off, self.v_off, self.freqs, batch.tok_seq,
-                          batch.tok_pos, table, entry.k_pages if write else None,
-                          entry.v_pages if write else None, s.n_heads, s.n_kv_heads, s.head_dim,
-                          s.value_dim, self.rotary_dim)
-        gate = proj[:, self.g_off:self.g_off + s.n_heads] if s.head_gate else None
+        q, gate = DA.rope_store(proj, self.q_off, self.k_off, self.v_off, self.g_off, self.freqs,
+                                batch.tok_seq, batch.tok_pos, table,
+                                entry.k_pages if write else None, entry.v_pages if write else None,
+                                s.n_heads, s.n_kv_heads, s.head_dim, s.value_dim, self.rotary_dim,
+                                self.rt.dtype, with_gate=s.head_gate)
 
         def finish(rows, then_norm, takes_halves):
             y = DA.attention(q, entry.k_pages, entry.v_pages, gate, batch, table, self.scale,

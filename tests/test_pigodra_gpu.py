@@ -29,13 +29,16 @@ def row_errors(got, want):
 def bf16_close(got, want):
     """A bfloat16 engine against float64 (or against itself, cut or batched another way, where
     other kernels round at other places).  Rows differ in how much they amplify a rounding
-    error (a head's result is divided by its own size, which may be small), so the bulk of the
-    rows is held to the tolerance and every row to a bound that a wrong key, a lost state or
-    a missing term would still break."""
-    e = row_errors(got, want)
-    if e.numel() < 20:               # a handful of rows has no bulk: the wide bound alone
-        return float(e.max()) < 0.35
-    return float(e.quantile(0.9)) < TOL_BF16 and float(e.max()) < 0.35
+    error: a head's result is divided by its own root mean square, which is small where the
+    two maps nearly cancel or the memory's answer nearly vanishes, and a row in a hundred may
+    amplify it fortyfold.  So nine rows in ten are held to the tolerance, and all but one in a
+    hundred (at least one) to a bound that a wrong key, a lost state or a missing term, which
+    touch most rows, would still break.  The float32 engine is the sharp test."""
+    e = row_errors(got, want).sort().values
+    rest = e[:max(1, e.numel() - max(1, e.numel() // 100))]
+    if float(rest.max()) >= 0.35:
+        return False
+    return e.numel() < 20 or float(e.quantile(0.9)) < TOL_BF16
 
 
 def close(got, want, dtype, tol):
@@ -202,20 +205,20 @@ def _attention_alone(dtype, H, G, dim, vdim, window, first, rot, lens, starts, b
             pos_of += list(range(lo, hi))
         if not seq_of:
             continue
-        proj = torch.cat(rows).contiguous()
+        proj = torch.cat(rows).float().contiguous()
         tok_seq = torch.tensor(seq_of, dtype=torch.int32, device=DEV)
         tok_pos = torch.tensor(pos_of, dtype=torch.int32, device=DEV)
-        q = DA.rope_store(proj, 0, k_off, v_off, freqs, tok_seq, tok_pos, table, k_pages, v_pages,
-                          H, G, dim, vdim, rot)
+        q, gate = DA.rope_store(proj, 0, k_off, v_off, g_off, freqs, tok_seq, tok_pos, table, k_pages,
+                                v_pages, H, G, dim, vdim, rot, dtype)
         if phase == 1 and kernel == "plain":
-            y = DA.attention_generic(q, k_pages, v_pages, proj[:, g_off:g_off + H], tok_seq, tok_pos,
+            y = DA.attention_generic(q, k_pages, v_pages, gate, tok_seq, tok_pos,
                                      table, scale, window, first, lam, eps, out_scale)
         elif phase == 1:
             # the matrix-core kernel; with one token per sequence also its form in which the
             # waves of a workgroup share the keys
             q_start = torch.tensor([sum(lens[:b]) for b in range(len(lens) + 1)], dtype=torch.int32, device=DEV)
             start_pos = torch.tensor(starts, dtype=torch.int32, device=DEV)
-            y = DA.attention_mfma(q, k_pages, v_pages, proj[:, g_off:g_off + H], q_start, start_pos,
+            y = DA.attention_mfma(q, k_pages, v_pages, gate, q_start, start_pos,
                                   table, len(lens), max(lens), scale, window, first, lam, eps, out_scale,
                                   single_tokens=kernel == "shared")
         if phase == 1:
