@@ -1,5 +1,6 @@
-"""An MI355X-native generation library for the Llama 2/3 dense decoder and the Pigodra stack
-(matrix-memory and differential-attention layers).
+"""An MI355X-native generation library for the Llama 2/3 dense decoder, the Pigodra stack
+(matrix-memory and differential-attention layers) and the Nizedra stack (lightning attention,
+latent attention, attention with mixed heads, looped layers).
 
 From a model folder (``config.json`` + safetensors) or seeded random weights to
 generated tokens, through hand-written HIP kernels for gfx950:
@@ -14,7 +15,7 @@ from .config.registry import (architecture, find_preset, known_architectures,
 from .engine.batch import Entry
 from .engine.step import Engine
 from .parts.base import (register_block, register_feed_forward, register_mixer, register_norm,
-                         register_position)
+                         register_position, register_stream_step)
 from .weights.random_init import write_random_model
 from .engine.generate import GenerationResult, generate
 from .engine.cli import main

@@ -35,6 +35,9 @@ class Architecture:
     describe: Callable[[object], dict] = None
     # the config.json key that holds the number of layers (a benchmark may run fewer)
     layer_count_key: str = "num_hidden_layers"
+    # (typed configuration, {tensor name: shape} of the folder's checkpoint) -> typed
+    # configuration, for sizes that only a tensor's shape gives
+    sizes_from_tensors: Callable[[object, dict], object] = None
 
     def layouts(self, config) -> tuple:
         """Every layout a checkpoint of ``config`` may have; the first is the one that
@@ -115,4 +118,15 @@ def read_model_folder(folder: str):
     with open(path) as f:
         raw = json.load(f)
     arch = architecture_of(raw)
-    return arch, arch.read_config(raw)
+    config = arch.read_config(raw)
+    if arch.sizes_from_tensors is not None:
+        from ..weights.safetensors_io import open_model_files
+        shapes = {}
+        try:
+            for f in open_model_files(folder):
+                shapes.update({name: shape for name, (_, shape) in f.entries.items()})
+        except FileNotFoundError:
+            shapes = None                 # a folder with a config.json only (presets, reports)
+        if shapes is not None:
+            config = arch.sizes_from_tensors(config, shapes)
+    return arch, config

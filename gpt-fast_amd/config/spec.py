@@ -108,6 +108,101 @@ class MatrixMemorySpec:
 
 
 @dataclass(frozen=True)
+class MixedHeadsAttentionSpec:
+    """Causal attention with grouped key/value heads whose scores are mixed across heads before
+    the softmax.  Projections of q, k, v and the output have biases if ``biases``; q and k are
+    divided by their root mean square over ``head_dim`` per head (``qk_norm_eps``; None: not
+    normed); then, for query i, key j <= i and head g,
+
+        s_g = (q_g . k_j) * scale * temperature[g]          (a learned number per head)
+        s_g = softcap * tanh(s_g / softcap)                 (if ``softcap``)
+        s_g = s_g + table[bucket(i - j), g]                 (if ``bias_rows``)
+        score_h = sum_g talk[h, g] s_g                      (if ``mix_heads``)
+
+    and head h's softmax over j weighs the values of kv head ``h // (H / G)``.  The distance
+    table has ``bias_rows`` rows: with ``half = bias_rows // 2``, distance n < half has its own
+    row n; further distances share rows in logarithmic steps,
+    ``half + floor(ln(n / half) / ln(bias_max / half) * (bias_rows - half))``, the last row
+    taking everything beyond."""
+    dim: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    value_dim: int
+    scale: float
+    softcap: Optional[float] = None
+    bias_rows: int = 0
+    bias_max: float = 0.0
+    qk_norm_eps: Optional[float] = None
+    head_temperature: bool = True
+    mix_heads: bool = True
+    biases: bool = True
+    kind: str = "mixed_heads_attention"
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose keys and values are expanded from one latent vector per token.  The
+    query goes through a latent of ``q_rank`` with an RMS norm, then up to ``n_heads`` heads of
+    ``head_dim`` plain and ``rot_dim`` rotated elements; one projection gives the token's
+    latent of ``kv_rank`` (RMS-normed) and one rotated key part of ``rot_dim`` that all heads
+    share; a head's plain key is ``w_uk`` of the latent, its value ``w_uv`` of it
+    (``value_dim``).  score = (q_plain . k_plain + q_rot . k_rot) * scale.  ``position``
+    rotates the first ``position.rotary_dim`` elements of the rotated parts.  ``window`` W:
+    keys at distance < W only.  The cache holds the latent and the rotated key part."""
+    dim: int
+    n_heads: int
+    head_dim: int
+    rot_dim: int
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    eps: float
+    position: PositionSpec
+    window: Optional[int] = None
+    kind: str = "latent_attention"
+
+
+@dataclass(frozen=True)
+class DecayedMemorySpec:
+    """Linear attention with a fixed decay per head (lightning attention): q, k (``key_dim``)
+    and v (``value_dim``) are silu of their projections; per head a float32 state
+    ``S [key_dim, value_dim]``, zero at a sequence's start: ``S' = decay_h S + k v^T``,
+    ``o = S'^T q``.  The heads' results side by side are RMS-normed as one row (``eps``, a
+    weight per element), multiplied by sigmoid of a gate projection and projected out."""
+    dim: int
+    n_heads: int
+    key_dim: int
+    value_dim: int
+    decay: Tuple[float, ...]
+    eps: float
+    kind: str = "decayed_memory"
+
+
+@dataclass(frozen=True)
+class DenseFeedForwardSpec:
+    """``w_down( act(w_up x) )`` without biases.  ``activation`` "xielu": with two learned
+    numbers p, q (the parameter ``act``): z > 0: ``softplus(p) z^2 + z/2``; z <= 0:
+    ``(1/2 + softplus(q)) (exp(z) - 1 - z) + z/2``.  Others: "silu", "gelu_tanh" (no
+    parameter)."""
+    dim: int
+    hidden: int
+    activation: str = "xielu"
+    kind: str = "dense"
+
+
+@dataclass(frozen=True)
+class InputMixSpec:
+    """A step on the residual stream that stands before a run: ``x <- W [x; x0]`` with
+    ``W [dim, 2 dim]`` (the columns for x first) and x0 the embedded rows of the step's tokens.
+    ``name`` is the tensor's name; runs that name the same spec share the matrix."""
+    dim: int
+    name: str
+    kind: str = "input_mix"
+
+
+@dataclass(frozen=True)
 class GatedFeedForwardSpec:
     """w2( act(w1 x) * (w3 x) ) without biases (reference model.py:219-227); ``activation``
     "silu" or "gelu_tanh"."""
@@ -133,6 +228,11 @@ class LayerSpec:
     mixer_norm_name: str = "mixer_norm"
     feed_forward_name: str = "feed_forward"
     feed_forward_norm_name: str = "feed_forward_norm"
+    # "sandwich_norm": a second norm on each sublayer's result, before it joins the stream
+    mixer_out_norm: Optional[NormSpec] = None
+    feed_forward_out_norm: Optional[NormSpec] = None
+    mixer_out_norm_name: str = "mixer_out_norm"
+    feed_forward_out_norm_name: str = "feed_forward_out_norm"
 
 
 @dataclass(frozen=True)
@@ -141,9 +241,11 @@ class Run:
     ``ModelPlan.layers``; a layer may be named by several entries (its weights are then
     used more than once).  ``cache`` names the cache entry the mixer reads and writes;
     it defaults to an entry of this run's own.  A run with ``cache_from`` = index of an
-    earlier run reads that run's cache and writes nothing."""
+    earlier run reads that run's cache and writes nothing.  ``enter`` is the spec of a step on
+    the residual stream that stands before this run (``InputMixSpec``), or None."""
     layer: int
     cache_from: Optional[int] = None
+    enter: object = None
 
 
 @dataclass

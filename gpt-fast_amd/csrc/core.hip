@@ -731,3 +731,215 @@ extern "C" int gfa_gemm_bf16_naive(const void* a, const void* w, float* out, int
     gemm_bf16_naive_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)a, (const bf16_t*)w, out, M, N, K);
     return GFA_LAUNCH_RESULT();
 }
+
+// --------------------------------------------------------------------------------------
+// A sublayer's result joins the stream through a norm of its own ("sandwich" blocks):
+//     res[r, :] += y[r, :] * rsqrt(mean(y[r, :]^2) + eps_y) * wy[:]
+// and, if next_w is given, the norm that reads the stream next in the same pass:
+//     out[r, :] = res[r, :] * rsqrt(mean(res[r, :]^2) + eps_n) * next_w[:]     (type T)
+// y is float (a product's float sums).  One workgroup per row; statistics in float.
+template <typename T>
+__global__ __launch_bounds__(256) void normed_add_kernel(
+        float* __restrict__ res, const float* __restrict__ y, const float* __restrict__ wy,
+        float eps_y, const float* __restrict__ next_w, float eps_n, T* __restrict__ out, int dim) {
+    __shared__ float scratch[16];
+    const size_t row = (size_t)blockIdx.x * dim;
+    const float* yr = y + row;
+    float* rr = res + row;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) ss = fmaf(yr[d], yr[d], ss);
+    ss = block_sum(ss, scratch);
+    const float ry = rsqrtf(ss / (float)dim + eps_y);
+    float sn = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) {
+        const float v = rr[d] + yr[d] * ry * wy[d];
+        rr[d] = v;
+        sn = fmaf(v, v, sn);
+    }
+    if (next_w == nullptr) return;
+    sn = block_sum(sn, scratch);
+    const float rn = rsqrtf(sn / (float)dim + eps_n);
+    T* o = out + row;
+    // every thread reads back only what it wrote itself
+    for (int d = threadIdx.x; d < dim; d += 256) store_from_float(o + d, rr[d] * rn * next_w[d]);
+}
+
+extern "C" int gfa_normed_add(float* res, const float* y, const float* wy, float eps_y,
+                              const float* next_w, float eps_n, void* out, int out_bf16,
+                              int n_rows, int dim, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (out_bf16)
+        normed_add_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(res, y, wy, eps_y, next_w, eps_n,
+                                                             (bf16_t*)out, dim);
+    else
+        normed_add_kernel<float><<<n_rows, 256, 0, stream>>>(res, y, wy, eps_y, next_w, eps_n,
+                                                            (float*)out, dim);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// Activations of a feed-forward without a gate, element by element, in float:
+//   0 silu, 1 gelu (tanh form), 2 xIELU with two numbers a = softplus(p), b = 1/2 + softplus(q):
+//     z > 0: a z^2 + z/2        z <= 0: b (exp(z) - 1 - z) + z/2
+template <int ACT>
+__device__ __forceinline__ float activation(float z, float a, float b) {
+    if (ACT == 0) return z / (1.f + expf(-z));
+    if (ACT == 1) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    return z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z);
+}
+
+template <typename T, int ACT>
+__global__ void activate_kernel(const T* __restrict__ x, T* __restrict__ out, size_t total,
+                                float a, float b) {
+    for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < total;
+         e += (size_t)gridDim.x * blockDim.x)
+        store_from_float(out + e, activation<ACT>(load_as_float(x + e), a, b));
+}
+
+// eight bfloat16 per thread
+template <int ACT>
+__global__ __launch_bounds__(256) void activate_bf16x8_kernel(const uint4* __restrict__ x,
+                                                              uint4* __restrict__ out, size_t total8,
+                                                              float a, float b) {
+    for (size_t e = blockIdx.x * (size_t)256 + threadIdx.x; e < total8; e += (size_t)gridDim.x * 256) {
+        uint4 v = x[e];
+        uint32_t* w = (uint32_t*)&v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float lo = activation<ACT>(__uint_as_float(w[i] << 16), a, b);
+            const float hi = activation<ACT>(__uint_as_float(w[i] & 0xffff0000u), a, b);
+            w[i] = (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+        }
+        out[e] = v;
+    }
+}
+
+template <int ACT>
+static int launch_activate(const void* x, void* out, size_t total, float a, float b, int is_bf16,
+                           hipStream_t stream) {
+    if (is_bf16 && total % 8 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+        const size_t n8 = total / 8;
+        const int blocks = (int)((n8 + 255) / 256 < 262144 ? (n8 + 255) / 256 : 262144);
+        activate_bf16x8_kernel<ACT><<<blocks, 256, 0, stream>>>((const uint4*)x, (uint4*)out, n8, a, b);
+        return GFA_LAUNCH_RESULT();
+    }
+    const int blocks = (int)((total + 255) / 256 < 262144 ? (total + 255) / 256 : 262144);
+    if (is_bf16)
+        activate_kernel<bf16_t, ACT><<<blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, total, a, b);
+    else
+        activate_kernel<float, ACT><<<blocks, 256, 0, stream>>>((const float*)x, (float*)out, total, a, b);
+    return GFA_LAUNCH_RESULT();
+}
+
+extern "C" int gfa_activate(const void* x, void* out, size_t total, int act, float a, float b,
+                            int is_bf16, hipStream_t stream) {
+    if (total == 0) return 0;
+    if (act == 0) return launch_activate<0>(x, out, total, a, b, is_bf16, stream);
+    if (act == 1) return launch_activate<1>(x, out, total, a, b, is_bf16, stream);
+    if (act == 2) return launch_activate<2>(x, out, total, a, b, is_bf16, stream);
+    return (int)hipErrorInvalidValue;
+}
+
+// --------------------------------------------------------------------------------------
+// out[r, :] = [a[r, :], b[r, :]] in type T from two float matrices of dim columns each: the
+// operand of a product over the stream and the embedded rows side by side.
+template <typename T>
+__global__ void concat_rows_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                   T* __restrict__ out, int dim) {
+    const size_t r = blockIdx.x;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        store_from_float(out + r * 2 * dim + d, a[r * dim + d]);
+        store_from_float(out + r * 2 * dim + dim + d, b[r * dim + d]);
+    }
+}
+
+extern "C" int gfa_concat_rows(const float* a, const float* b, void* out, int out_bf16, int n_rows,
+                               int dim, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (out_bf16) concat_rows_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(a, b, (bf16_t*)out, dim);
+    else concat_rows_kernel<float><<<n_rows, 256, 0, stream>>>(a, b, (float*)out, dim);
+    return GFA_LAUNCH_RESULT();
+}
+
+// res[r, :] += bias[:]
+__global__ void add_bias_kernel(float* __restrict__ res, const float* __restrict__ bias, int dim) {
+    const size_t r = blockIdx.x;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) res[r * dim + d] += bias[d];
+}
+
+extern "C" int gfa_add_bias(float* res, const float* bias, int n_rows, int dim, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    add_bias_kernel<<<n_rows, 256, 0, stream>>>(res, bias, dim);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// A batch of float32 products with strides: for every b < B
+//     out[b][m, n] = sum_k a[b][m, k] * w[b][n, k]
+// with element (m, k) of a[b] at a + b sab + m sam + k (unit stride along k), element (n, k)
+// of w[b] at w + b swb + n swn + k swk, element (m, n) of out[b] at out + b sob + m som + n.
+// The same tiles and the same chain of fused multiply-adds per output as gemm_f32_kernel.
+__global__ __launch_bounds__(256) void gemm_f32_strided_kernel(
+        const float* __restrict__ a, const float* __restrict__ w, float* __restrict__ out,
+        int M, int N, int K, long long sab, long long sam, long long swb, long long swn,
+        long long swk, long long sob, long long som) {
+    __shared__ float As[GF_BK][GF_BM + 4];
+    __shared__ float Ws[GF_BK][GF_BN + 4];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int m0 = blockIdx.y * GF_BM, n0 = blockIdx.x * GF_BN;
+    a += (size_t)blockIdx.z * sab;
+    w += (size_t)blockIdx.z * swb;
+    out += (size_t)blockIdx.z * sob;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += GF_BK) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = threadIdx.x + i * 256;
+            const int r = e >> 4, c = e & 15;
+            const int k = k0 + c;
+            const int m = m0 + r, n = n0 + r;
+            As[c][r] = (m < M && k < K) ? a[(size_t)m * sam + k] : 0.f;
+            Ws[c][r] = (n < N && k < K) ? w[(size_t)n * swn + (size_t)k * swk] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < GF_BK; ++kk) {
+            float av[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wv[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n < N) out[(size_t)m * som + n] = acc[i][j];
+        }
+    }
+}
+
+extern "C" int gfa_gemm_f32_strided(const float* a, const float* w, float* out, int B, int M, int N,
+                                    int K, long long sab, long long sam, long long swb,
+                                    long long swn, long long swk, long long sob, long long som,
+                                    hipStream_t stream) {
+    if (B <= 0 || M <= 0 || N <= 0) return 0;
+    if (B > 65535 || (M + GF_BM - 1) / GF_BM > 65535) return (int)hipErrorInvalidValue;
+    dim3 grid((N + GF_BN - 1) / GF_BN, (M + GF_BM - 1) / GF_BM, B);
+    gemm_f32_strided_kernel<<<grid, 256, 0, stream>>>(a, w, out, M, N, K, sab, sam, swb, swn, swk,
+                                                      sob, som);
+    return GFA_LAUNCH_RESULT();
+}

@@ -1,0 +1,432 @@
+// Attention over the paged cache whose scores take further steps between the dot product and
+// the softmax, and whose keys and values may have different sizes; all arithmetic in float.
+//
+// For the token at position i of a sequence, head h (kv head g = h / (H / G)) and key j with
+// max(0, i - window + 1) <= j <= i (window 0: from 0):
+//     s_h(j) = (q_h . k_g(j)) * scale * temperature[h]                  (temperature optional)
+//     s_h(j) = softcap * tanh(s_h(j) / softcap)                         (softcap > 0)
+//     s_h(j) = s_h(j) + bias[row(i - j), h]                             (bias optional)
+//     z_h(j) = sum_h' talk[h, h'] s_h'(j)                               (talk optional)
+//     out_h  = sum_j softmax_j(z_h)(j) v_g(j)
+// row(n) = lookup[n] for n < n_lookup, else bias_rows - 1 (the host fills the lookup table).
+//
+// The cache keeps keys and values in the orders of common.h (key_offset, value_offset) with
+// head sizes hd for keys and vd for values.  q and out are addressed by strides, so rows may
+// lie token by token or head by head.
+//
+// Also here: the kernels that make q, keys and values of two mixers from their projections'
+// float sums and put keys and values into the cache (unit-norm heads with biases; a normed
+// latent with one rotated key part).
+#include "common.h"
+
+#define SA_THREADS 256
+#define SA_WAVES 4
+
+struct SAShape {
+    int H, G, hd, vd;
+    long long q_tok, q_head, o_tok, o_head;      // strides in elements
+    int table_stride, window;
+    float scale, softcap;
+    int bias_rows, n_lookup;
+};
+
+template <typename T> struct Pack8;
+template <> struct Pack8<bf16_t> {
+    uint4 raw;
+    __device__ __forceinline__ void load(const bf16_t* p) { raw = *(const uint4*)p; }
+    __device__ __forceinline__ float get(int i) const {
+        const uint32_t w = ((const uint32_t*)&raw)[i >> 1];
+        return (i & 1) ? __uint_as_float(w & 0xffff0000u) : __uint_as_float(w << 16);
+    }
+};
+template <> struct Pack8<float> {
+    float4 a, b;
+    __device__ __forceinline__ void load(const float* p) {
+        a = *(const float4*)p;
+        b = *(const float4*)(p + 4);
+    }
+    __device__ __forceinline__ float get(int i) const {
+        return i < 4 ? ((const float*)&a)[i] : ((const float*)&b)[i - 4];
+    }
+};
+
+// One workgroup per (token, block of 4 * HPW heads): wave w owns heads w, w + 4, ... of the
+// block; a lane is a key of the page for the scores and a value element for the sums.  Keys
+// are walked a page at a time, pages counted from the sequence's start, so a token's result
+// does not depend on how its sequence was cut into steps.
+template <typename T, int HPW, int VPT>
+__global__ __launch_bounds__(SA_THREADS) void scored_attention_kernel(
+        const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+        const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+        const int* __restrict__ table, const float* __restrict__ temperature,
+        const float* __restrict__ bias, const int* __restrict__ lookup,
+        const float* __restrict__ talk, T* __restrict__ out, SAShape s) {
+    extern __shared__ __attribute__((aligned(16))) float sa_lds[];
+    constexpr int HB = SA_WAVES * HPW;
+    float* qs = sa_lds;                          // [HB][hd]
+    float* sc = qs + HB * s.hd;                  // [HB][64] scores before the mix
+    float* pr = sc + HB * GFA_PAGE;              // [HB][64] softmax weights
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = blockIdx.x, h0 = blockIdx.y * HB;
+    const int pos = tok_pos[n];
+    const int* pages = table + (size_t)tok_seq[n] * s.table_stride;
+    const int lo = (s.window > 0 && pos - s.window + 1 > 0) ? pos - s.window + 1 : 0;
+    const int per_group = s.H / s.G;
+
+    for (int e = threadIdx.x; e < HB * s.hd; e += SA_THREADS) {
+        const int hl = e / s.hd, d = e - hl * s.hd;
+        qs[e] = (h0 + hl < s.H)
+            ? load_as_float(q + (size_t)n * s.q_tok + (size_t)(h0 + hl) * s.q_head + d) : 0.f;
+    }
+    float m[HPW], l[HPW], acc[HPW][VPT];
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+        m[i] = -INFINITY;
+        l[i] = 0.f;
+#pragma unroll
+        for (int e = 0; e < VPT; ++e) acc[i][e] = 0.f;
+    }
+    __syncthreads();
+
+    for (int pg = lo / GFA_PAGE; pg <= pos / GFA_PAGE; ++pg) {
+        const int page = pages[pg];
+        const int j = pg * GFA_PAGE + lane;
+        const bool seen = j >= lo && j <= pos;
+        float z[HPW];
+#pragma unroll
+        for (int i = 0; i < HPW; ++i) {
+            const int hl = wave + SA_WAVES * i, h = h0 + hl;
+            z[i] = 0.f;
+            if (h >= s.H || !seen) continue;
+            const int g = h / per_group;
+            const T* kr = k_pages + cache_region(page, g, s.G, s.hd);
+            const float* qh = qs + hl * s.hd;
+            float dot = 0.f;
+            if (s.hd % 8 == 0) {
+                for (int d = 0; d < s.hd; d += 8) {
+                    Pack8<T> kk;
+                    kk.load(kr + key_offset(lane, d, s.hd));
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) dot = fmaf(qh[d + t], kk.get(t), dot);
+                }
+            } else {
+                for (int d = 0; d < s.hd; ++d)
+                    dot = fmaf(qh[d], load_as_float(kr + key_offset(lane, d, s.hd)), dot);
+            }
+            float v = dot * s.scale;
+            if (temperature) v *= temperature[h];
+            if (s.softcap > 0.f) v = s.softcap * tanhf(v / s.softcap);
+            if (bias) {
+                const int dist = pos - j;
+                const int row = dist < s.n_lookup ? lookup[dist] : s.bias_rows - 1;
+                v += bias[(size_t)row * s.H + h];
+            }
+            z[i] = v;
+        }
+        if (talk) {
+#pragma unroll
+            for (int i = 0; i < HPW; ++i) sc[(wave + SA_WAVES * i) * GFA_PAGE + lane] = z[i];
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < HPW; ++i) {
+                const int h = wave + SA_WAVES * i;           // talk: one block holds every head
+                if (h >= s.H) continue;
+                float v = 0.f;
+                for (int g = 0; g < s.H; ++g) v = fmaf(talk[h * s.H + g], sc[g * GFA_PAGE + lane], v);
+                z[i] = v;
+            }
+        }
+        float alpha[HPW];
+#pragma unroll
+        for (int i = 0; i < HPW; ++i) {
+            const int hl = wave + SA_WAVES * i;
+            const float v = seen ? z[i] : -INFINITY;
+            const float m_new = fmaxf(m[i], wave_max(v));
+            alpha[i] = m_new == -INFINITY ? 1.f : expf(m[i] - m_new);
+            const float p = seen ? expf(v - m_new) : 0.f;
+            l[i] = l[i] * alpha[i] + wave_sum(p);
+            m[i] = m_new;
+            pr[hl * GFA_PAGE + lane] = p;
+        }
+        __syncthreads();
+        // keys of this page that are seen: [j_lo, j_hi], in groups of eight
+        const int j_lo = lo > pg * GFA_PAGE ? lo - pg * GFA_PAGE : 0;
+        const int j_hi = pos - pg * GFA_PAGE < GFA_PAGE - 1 ? pos - pg * GFA_PAGE : GFA_PAGE - 1;
+#pragma unroll
+        for (int i = 0; i < HPW; ++i) {
+            const int hl = wave + SA_WAVES * i, h = h0 + hl;
+            if (h >= s.H) continue;
+            const int g = h / per_group;
+            const T* vr = v_pages + cache_region(page, g, s.G, s.vd);
+            const float* ph = pr + hl * GFA_PAGE;
+#pragma unroll
+            for (int e = 0; e < VPT; ++e) {
+                const int d = lane + 64 * e;
+                float a = acc[i][e] * alpha[i];
+                if (d < s.vd) {
+                    for (int kg = j_lo >> 3; kg <= j_hi >> 3; ++kg) {
+                        Pack8<T> vv;
+                        vv.load(vr + value_offset(d, kg * 8, s.vd));
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) {
+                            const int key = kg * 8 + t;
+                            // the pool is not cleared: what lies beyond the seen keys may be anything
+                            const float val = (key >= j_lo && key <= j_hi) ? vv.get(t) : 0.f;
+                            a = fmaf(ph[key], val, a);
+                        }
+                    }
+                }
+                acc[i][e] = a;
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+        const int h = h0 + wave + SA_WAVES * i;
+        if (h >= s.H) continue;
+        T* o = out + (size_t)n * s.o_tok + (size_t)h * s.o_head;
+#pragma unroll
+        for (int e = 0; e < VPT; ++e) {
+            const int d = lane + 64 * e;
+            if (d < s.vd) store_from_float(o + d, acc[i][e] / l[i]);
+        }
+    }
+}
+
+template <typename T, int HPW, int VPT>
+static int sa_launch(const void* q, const void* k_pages, const void* v_pages, const int* tok_seq,
+                     const int* tok_pos, const int* table, const float* temperature,
+                     const float* bias, const int* lookup, const float* talk, void* out,
+                     int n_tokens, const SAShape& s, hipStream_t stream) {
+    constexpr int HB = SA_WAVES * HPW;
+    const size_t shmem = (size_t)HB * (s.hd + 2 * GFA_PAGE) * sizeof(float);
+    if (shmem > 64 * 1024) return (int)hipErrorInvalidValue;
+    dim3 grid(n_tokens, (s.H + HB - 1) / HB);
+    scored_attention_kernel<T, HPW, VPT><<<grid, SA_THREADS, shmem, stream>>>(
+        (const T*)q, (const T*)k_pages, (const T*)v_pages, tok_seq, tok_pos, table, temperature,
+        bias, lookup, talk, (T*)out, s);
+    return GFA_LAUNCH_RESULT();
+}
+
+template <typename T>
+static int sa_dispatch(const void* q, const void* k_pages, const void* v_pages, const int* tok_seq,
+                       const int* tok_pos, const int* table, const float* temperature,
+                       const float* bias, const int* lookup, const float* talk, void* out,
+                       int n_tokens, const SAShape& s, hipStream_t stream) {
+    // heads per wave: with a mix one workgroup holds every head; without, one head per wave
+    const int hpw = talk ? (s.H + SA_WAVES - 1) / SA_WAVES : 1;
+    const int vpt = (s.vd + 63) / 64;
+#define SA_GO(HPW, VPT) return sa_launch<T, HPW, VPT>(q, k_pages, v_pages, tok_seq, tok_pos, table, \
+        temperature, bias, lookup, talk, out, n_tokens, s, stream)
+    if (hpw <= 1) {
+        if (vpt <= 2) SA_GO(1, 2);
+        if (vpt <= 8) SA_GO(1, 8);
+    } else if (hpw <= 4) {
+        if (vpt <= 2) SA_GO(4, 2);
+        if (vpt <= 8) SA_GO(4, 8);
+    } else if (hpw <= 16) {
+        if (vpt <= 2) SA_GO(16, 2);
+    }
+#undef SA_GO
+    return (int)hipErrorInvalidValue;
+}
+
+extern "C" int gfa_scored_attention(const void* q, const void* k_pages, const void* v_pages,
+                                    const int* tok_seq, const int* tok_pos, const int* table,
+                                    int table_stride, const float* temperature, const float* bias,
+                                    const int* lookup, const float* talk, void* out, int n_tokens,
+                                    int H, int G, int hd, int vd, long long q_tok, long long q_head,
+                                    long long o_tok, long long o_head, float scale, float softcap,
+                                    int bias_rows, int n_lookup, int window, int is_bf16,
+                                    hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (G <= 0 || H % G || hd <= 0 || vd <= 0 || vd > 512) return (int)hipErrorInvalidValue;
+    SAShape s{H, G, hd, vd, q_tok, q_head, o_tok, o_head, table_stride, window, scale, softcap,
+              bias_rows, n_lookup};
+    if (is_bf16)
+        return sa_dispatch<bf16_t>(q, k_pages, v_pages, tok_seq, tok_pos, table, temperature, bias,
+                                   lookup, talk, out, n_tokens, s, stream);
+    return sa_dispatch<float>(q, k_pages, v_pages, tok_seq, tok_pos, table, temperature, bias,
+                              lookup, talk, out, n_tokens, s, stream);
+}
+
+// --------------------------------------------------------------------------------------
+// q, keys and values of attention with unit-norm heads from the projection's float sums:
+// a row of proj is [H heads of q | G heads of k | G heads of v] (d, d, dv wide); the bias
+// (same layout, optional) is added first; every head of q and k is divided by its root mean
+// square (eps inside the root; eps < 0: not normed).  q goes to q_out [N, H, d]; keys and
+// values to the token's place in the cache (skipped if k_pages is null).  One workgroup per
+// token, one wave per head vector, float arithmetic, one rounding at the store.
+template <typename T>
+__global__ __launch_bounds__(SA_THREADS) void unit_heads_store_kernel(
+        const float* __restrict__ proj, int row_width, const float* __restrict__ bias,
+        T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
+        const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+        const int* __restrict__ table, int table_stride, int H, int G, int d, int dv, float eps) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = blockIdx.x;
+    const float* row = proj + (size_t)n * row_width;
+    const int pos = tok_pos[n];
+    const int page = k_pages ? table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE] : 0;
+    const int slot = pos % GFA_PAGE;
+    for (int u = wave; u < H + 2 * G; u += SA_WAVES) {
+        const bool is_q = u < H, is_k = !is_q && u < H + G;
+        const int width = (is_q || is_k) ? d : dv;
+        const int off = is_q ? u * d : (is_k ? H * d + (u - H) * d : (H + G) * d + (u - H - G) * dv);
+        if (!is_q && !k_pages) continue;
+        float r = 1.f;
+        if ((is_q || is_k) && eps >= 0.f) {
+            float ss = 0.f;
+            for (int e = lane; e < width; e += 64) {
+                const float x = row[off + e] + (bias ? bias[off + e] : 0.f);
+                ss = fmaf(x, x, ss);
+            }
+            r = rsqrtf(wave_sum(ss) / (float)width + eps);
+        }
+        for (int e = lane; e < width; e += 64) {
+            const float x = (row[off + e] + (bias ? bias[off + e] : 0.f)) * r;
+            if (is_q) store_from_float(q_out + ((size_t)n * H + u) * d + e, x);
+            else if (is_k) store_from_float(k_pages + key_elem(page, u - H, slot, e, G, d), x);
+            else store_from_float(v_pages + value_elem(page, u - H - G, e, slot, G, dv), x);
+        }
+    }
+}
+
+extern "C" int gfa_unit_heads_store(const float* proj, int row_width, const float* bias, void* q_out,
+                                    void* k_pages, void* v_pages, const int* tok_seq,
+                                    const int* tok_pos, const int* table, int table_stride,
+                                    int n_tokens, int H, int G, int d, int dv, float eps,
+                                    int is_bf16, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (is_bf16)
+        unit_heads_store_kernel<bf16_t><<<n_tokens, SA_THREADS, 0, stream>>>(
+            proj, row_width, bias, (bf16_t*)q_out, (bf16_t*)k_pages, (bf16_t*)v_pages, tok_seq,
+            tok_pos, table, table_stride, H, G, d, dv, eps);
+    else
+        unit_heads_store_kernel<float><<<n_tokens, SA_THREADS, 0, stream>>>(
+            proj, row_width, bias, (float*)q_out, (float*)k_pages, (float*)v_pages, tok_seq,
+            tok_pos, table, table_stride, H, G, d, dv, eps);
+    return GFA_LAUNCH_RESULT();
+}
+
+// --------------------------------------------------------------------------------------
+// The latents of latent attention from the float sums of the token's two down projections:
+// a row of proj is [q latent (q_rank) | kv latent (R) | key part to rotate (dr)].
+//   cq_out[n, :] = rmsnorm(q latent) * wq              (operand of the query's up projection)
+//   c = rmsnorm(kv latent) * wkv  -> the cache's key elements 0 .. R-1 and value elements 0 .. R-1
+//   rotated part: pairs (2i, 2i+1), i < rotary_dim / 2, turned by pos * freqs[i], the rest as
+//   it is -> the cache's key elements R .. R+dr-1
+// The cache has one kv head with keys of R + dr and values of R.  One workgroup per token.
+template <typename T>
+__global__ __launch_bounds__(SA_THREADS) void latent_store_kernel(
+        const float* __restrict__ proj, int row_width, int q_rank, int R, int dr,
+        const float* __restrict__ wq, const float* __restrict__ wkv, float eps,
+        const float* __restrict__ freqs, int rotary_dim, T* __restrict__ cq_out,
+        T* __restrict__ k_pages, T* __restrict__ v_pages, const int* __restrict__ tok_seq,
+        const int* __restrict__ tok_pos, const int* __restrict__ table, int table_stride) {
+    __shared__ float scratch[16];
+    const int n = blockIdx.x;
+    const float* row = proj + (size_t)n * row_width;
+    const int pos = tok_pos[n];
+    float ss = 0.f;
+    for (int e = threadIdx.x; e < q_rank; e += SA_THREADS) ss = fmaf(row[e], row[e], ss);
+    const float rq = rsqrtf(block_sum(ss, scratch) / (float)q_rank + eps);
+    for (int e = threadIdx.x; e < q_rank; e += SA_THREADS)
+        store_from_float(cq_out + (size_t)n * q_rank + e, row[e] * rq * wq[e]);
+    if (!k_pages) return;
+    const float* kv = row + q_rank;
+    ss = 0.f;
+    for (int e = threadIdx.x; e < R; e += SA_THREADS) ss = fmaf(kv[e], kv[e], ss);
+    const float rc = rsqrtf(block_sum(ss, scratch) / (float)R + eps);
+    const int page = table[(size_t)tok_seq[n] * table_stride + pos / GFA_PAGE];
+    const int slot = pos % GFA_PAGE;
+    const int hd = R + dr;
+    for (int e = threadIdx.x; e < R; e += SA_THREADS) {
+        const float c = kv[e] * rc * wkv[e];
+        store_from_float(k_pages + key_elem(page, 0, slot, e, 1, hd), c);
+        store_from_float(v_pages + value_elem(page, 0, e, slot, 1, R), c);
+    }
+    const float* kr = kv + R;
+    for (int i = threadIdx.x; i < dr / 2; i += SA_THREADS) {
+        float u = kr[2 * i], v = kr[2 * i + 1];
+        if (2 * i < rotary_dim) {
+            float sn, cs;
+            sincosf((float)pos * freqs[i], &sn, &cs);
+            const float u2 = u * cs - v * sn, v2 = v * cs + u * sn;
+            u = u2;
+            v = v2;
+        }
+        store_from_float(k_pages + key_elem(page, 0, slot, R + 2 * i, 1, hd), u);
+        store_from_float(k_pages + key_elem(page, 0, slot, R + 2 * i + 1, 1, hd), v);
+    }
+    if ((dr & 1) && threadIdx.x == 0)
+        store_from_float(k_pages + key_elem(page, 0, slot, hd - 1, 1, hd), kr[dr - 1]);
+}
+
+extern "C" int gfa_latent_store(const float* proj, int row_width, int q_rank, int R, int dr,
+                                const float* wq, const float* wkv, float eps, const float* freqs,
+                                int rotary_dim, void* cq_out, void* k_pages, void* v_pages,
+                                const int* tok_seq, const int* tok_pos, const int* table,
+                                int table_stride, int n_tokens, int is_bf16, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (rotary_dim % 2 || rotary_dim > dr) return (int)hipErrorInvalidValue;
+    if (is_bf16)
+        latent_store_kernel<bf16_t><<<n_tokens, SA_THREADS, 0, stream>>>(
+            proj, row_width, q_rank, R, dr, wq, wkv, eps, freqs, rotary_dim, (bf16_t*)cq_out,
+            (bf16_t*)k_pages, (bf16_t*)v_pages, tok_seq, tok_pos, table, table_stride);
+    else
+        latent_store_kernel<float><<<n_tokens, SA_THREADS, 0, stream>>>(
+            proj, row_width, q_rank, R, dr, wq, wkv, eps, freqs, rotary_dim, (float*)cq_out,
+            (float*)k_pages, (float*)v_pages, tok_seq, tok_pos, table, table_stride);
+    return GFA_LAUNCH_RESULT();
+}
+
+// The query of latent attention from the float sums of its up projection, a row of
+// [H heads of (d plain | dr to rotate)]: the plain parts go head by head to
+// plain_out [H, N, d] (operand of the product with the keys' up projection), the rotated
+// parts to elements R .. R+dr-1 of full_out [H, N, R + dr], whose first R elements that
+// product fills.  grid (tokens, heads).
+template <typename T>
+__global__ void latent_query_kernel(const float* __restrict__ q, const float* __restrict__ freqs,
+                                    int rotary_dim, const int* __restrict__ tok_pos,
+                                    T* __restrict__ plain_out, T* __restrict__ full_out, int N, int H,
+                                    int d, int dr, int R) {
+    const int n = blockIdx.x, h = blockIdx.y;
+    const float* row = q + ((size_t)n * H + h) * (d + dr);
+    T* plain = plain_out + ((size_t)h * N + n) * d;
+    for (int e = threadIdx.x; e < d; e += blockDim.x) store_from_float(plain + e, row[e]);
+    T* full = full_out + ((size_t)h * N + n) * (R + dr) + R;
+    const float* qr = row + d;
+    const int pos = tok_pos[n];
+    for (int i = threadIdx.x; i < dr / 2; i += blockDim.x) {
+        float u = qr[2 * i], v = qr[2 * i + 1];
+        if (2 * i < rotary_dim) {
+            float sn, cs;
+            sincosf((float)pos * freqs[i], &sn, &cs);
+            const float u2 = u * cs - v * sn, v2 = v * cs + u * sn;
+            u = u2;
+            v = v2;
+        }
+        store_from_float(full + 2 * i, u);
+        store_from_float(full + 2 * i + 1, v);
+    }
+    if ((dr & 1) && threadIdx.x == 0) store_from_float(full + dr - 1, qr[dr - 1]);
+}
+
+extern "C" int gfa_latent_query(const float* q, const float* freqs, int rotary_dim,
+                                const int* tok_pos, void* plain_out, void* full_out, int n_tokens,
+                                int H, int d, int dr, int R, int is_bf16, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (H > 65535 || rotary_dim % 2 || rotary_dim > dr) return (int)hipErrorInvalidValue;
+    dim3 grid(n_tokens, H);
+    if (is_bf16)
+        latent_query_kernel<bf16_t><<<grid, 64, 0, stream>>>(q, freqs, rotary_dim, tok_pos,
+                                                             (bf16_t*)plain_out, (bf16_t*)full_out,
+                                                             n_tokens, H, d, dr, R);
+    else
+        latent_query_kernel<float><<<grid, 64, 0, stream>>>(q, freqs, rotary_dim, tok_pos,
+                                                            (float*)plain_out, (float*)full_out,
+                                                            n_tokens, H, d, dr, R);
+    return GFA_LAUNCH_RESULT();
+}

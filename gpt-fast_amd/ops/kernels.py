@@ -294,6 +294,103 @@ def add_rmsnorm(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, e
     return out
 
 
+def normed_add(residual: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float,
+               next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0,
+               out_dtype: Optional[torch.dtype] = None):
+    """residual += y * rsqrt(mean(y^2) + eps) * weight, row by row (a sublayer's result joins
+    the stream through a norm of its own); with ``next_weight`` also returns the RMS norm of
+    the new rows, ``residual * rsqrt(mean(residual^2) + next_eps) * next_weight`` in
+    ``out_dtype``, from the same pass.  residual and y float32 [N, D]; weights float32 [D]."""
+    require_device(residual, y, weight, next_weight)
+    require_contiguous(residual=residual, y=y, weight=weight, next_weight=next_weight)
+    _want(residual, torch.float32, "residual")
+    _want(y, torch.float32, "y")
+    _want(weight, torch.float32, "norm weight")
+    if residual.dim() != 2 or y.shape != residual.shape or weight.numel() != residual.shape[1]:
+        raise KernelError("normed_add: shapes of residual, y and the norm weight do not fit")
+    out = None
+    if next_weight is not None:
+        _want(next_weight, torch.float32, "next norm weight")
+        if next_weight.numel() != residual.shape[1] or out_dtype not in (torch.float32, torch.bfloat16):
+            raise KernelError("normed_add: the next norm's weight or output type does not fit")
+        out = torch.empty(residual.shape, dtype=out_dtype, device=residual.device)
+    check(library("core").gfa_normed_add(
+        ptr(residual), ptr(y), ptr(weight), _f(eps), ptr(next_weight), _f(next_eps), ptr(out),
+        _i(int(out is not None and out.dtype == torch.bfloat16)), _i(residual.shape[0]),
+        _i(residual.shape[1]), stream_handle()), "normed_add")
+    return out
+
+
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "xielu": 2}
+
+
+def activate(x: torch.Tensor, activation: str, a: float = 0.0, b: float = 0.0,
+             out: Optional[torch.Tensor] = None):
+    """out = act(x) element by element (float arithmetic, x's type): "silu", "gelu_tanh", or
+    "xielu" with its two numbers: z > 0: a z^2 + z/2; z <= 0: b (exp(z) - 1 - z) + z/2."""
+    require_device(x, out)
+    require_contiguous(x=x, out=out)
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"activation '{activation}': {sorted(ACTIVATIONS)}")
+    if out is None:
+        out = torch.empty_like(x)
+    elif out.shape != x.shape or out.dtype != x.dtype:
+        raise KernelError("activate: out must have x's shape and type")
+    check(library("core").gfa_activate(ptr(x), ptr(out), _sz(x.numel()), _i(ACTIVATIONS[activation]),
+                                       _f(a), _f(b), _i(_is_bf16(x)), stream_handle()), "activate")
+    return out
+
+
+def concat_rows(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype):
+    """[N, 2D] in ``out_dtype``: the rows of float32 a and b [N, D] side by side."""
+    require_device(a, b)
+    require_contiguous(a=a, b=b)
+    _want(a, torch.float32, "a")
+    _want(b, torch.float32, "b")
+    if a.dim() != 2 or a.shape != b.shape or out_dtype not in (torch.float32, torch.bfloat16):
+        raise KernelError("concat_rows: a and b must be float32 [N, D]")
+    out = torch.empty((a.shape[0], 2 * a.shape[1]), dtype=out_dtype, device=a.device)
+    check(library("core").gfa_concat_rows(ptr(a), ptr(b), ptr(out), _i(int(out_dtype == torch.bfloat16)),
+                                          _i(a.shape[0]), _i(a.shape[1]), stream_handle()), "concat_rows")
+    return out
+
+
+def add_bias(residual: torch.Tensor, bias: torch.Tensor):
+    """residual[r, :] += bias, float32."""
+    require_device(residual, bias)
+    require_contiguous(residual=residual, bias=bias)
+    _want(residual, torch.float32, "residual")
+    _want(bias, torch.float32, "bias")
+    if residual.dim() != 2 or bias.numel() != residual.shape[1]:
+        raise KernelError("add_bias: residual [N, D] and bias [D]")
+    check(library("core").gfa_add_bias(ptr(residual), ptr(bias), _i(residual.shape[0]),
+                                       _i(residual.shape[1]), stream_handle()), "add_bias")
+    return residual
+
+
+def gemm_f32_batched(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
+    """out[b] = a[b] w[b]^T for every b, float32: a [B, M, K] with unit stride along k,
+    w [B, N, K] with any strides, out [B, M, N] with unit stride along n (views allowed)."""
+    require_device(a, w, out)
+    for name, t in (("a", a), ("w", w), ("out", out)):
+        _want(t, torch.float32, name)
+        if t.dim() != 3:
+            raise KernelError(f"gemm_f32_batched: {name} must have three dimensions")
+    B, M, K_ = a.shape
+    N = w.shape[1]
+    if w.shape[0] != B or w.shape[2] != K_ or tuple(out.shape) != (B, M, N):
+        raise KernelError(f"gemm_f32_batched: a {tuple(a.shape)}, w {tuple(w.shape)} and out "
+                          f"{tuple(out.shape)} do not fit")
+    if (K_ > 1 and a.stride(2) != 1) or (N > 1 and out.stride(2) != 1):
+        raise KernelError("gemm_f32_batched: a and out need unit stride in their last dimension")
+    ll = ctypes.c_longlong
+    check(library("core").gfa_gemm_f32_strided(
+        ptr(a), ptr(w), ptr(out), _i(B), _i(M), _i(N), _i(K_), ll(a.stride(0)), ll(a.stride(1)),
+        ll(w.stride(0)), ll(w.stride(1)), ll(w.stride(2)), ll(out.stride(0)), ll(out.stride(1)),
+        stream_handle()), "gemm_f32_batched")
+    return out
+
+
 # ----------------------------------------------------------------------------- sampling
 # vocabularies beyond this are spread over many workgroups per row
 SPLIT_SAMPLING_ABOVE = 16384

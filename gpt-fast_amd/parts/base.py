@@ -14,6 +14,8 @@ Interfaces (N = tokens of the step, D = model width):
 * feed-forward:  ``forward(x [N, D], batch, residual)`` adds its output into ``residual``
 * position:      ``rotate_and_store(qkv, batch, entry, n_heads, n_kv_heads, head_dim) -> q``
 * block:         ``forward(residual, batch, entry)`` updates ``residual`` in place
+* stream step:   ``forward(residual float32 [N, D], embedded float32 [N, D], batch) ->`` the new
+                 stream, float32 [N, D] (a step that a plan puts before a run, ``Run.enter``)
 
 A new part is a class with these methods, registered under a new ``kind``; its spec is
 any object with that ``kind`` attribute.
@@ -159,6 +161,7 @@ POSITIONS = _Registry("position encoding")
 MIXERS = _Registry("mixer")
 FEED_FORWARDS = _Registry("feed-forward")
 BLOCKS = _Registry("block arrangement")      # keyed by LayerSpec.arrangement
+STREAM_STEPS = _Registry("stream step")      # what a plan's Run.enter names
 
 
 def register_norm(kind, factory):
@@ -179,6 +182,10 @@ def register_feed_forward(kind, factory):
 
 def register_block(arrangement, factory):
     return BLOCKS.register(arrangement, factory)
+
+
+def register_stream_step(kind, factory):
+    return STREAM_STEPS.register(kind, factory)
 
 
 def check_bound(owner: str, declared: Dict[str, Param], tensors: Dict[str, torch.Tensor]) -> None:

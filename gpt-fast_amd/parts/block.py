@@ -1,5 +1,8 @@
 """How norms, mixer, feed-forward and the residual stream are wired in one layer."""
+import torch
+
 from ..config.spec import LayerSpec
+from ..ops import kernels as K
 from .base import FEED_FORWARDS, MIXERS, NORMS, Part, ResidualStream, Runtime, register_block
 
 
@@ -79,4 +82,60 @@ class PreNormBlock(Part):
             stream.tensor                    # a caller with a plain tensor gets the sums now
 
 
+class SandwichNormBlock(PreNormBlock):
+    """``h = x + norm1b(mixer(norm1(x))); out = h + norm2b(ffn(norm2(h)))``: a norm before
+    each sublayer and a second one on its result, before that joins the stream.  A sublayer
+    adds into a float32 tensor of its own, which starts at zero; one kernel then norms it,
+    adds it to the stream and, where the block knows which norm reads the stream next (its
+    own feed-forward's), applies that one in the same pass."""
+
+    takes_stream = False
+    takes_prepared = False
+
+    def __init__(self, spec: LayerSpec, runtime: Runtime):
+        super().__init__(spec, runtime)
+        if spec.mixer_out_norm is None or (spec.feed_forward is not None
+                                           and spec.feed_forward_out_norm is None):
+            raise ValueError("a sandwich_norm block needs a norm on each sublayer's result")
+        self.rt = runtime
+        self.mixer_out_norm = NORMS.build(spec.mixer_out_norm, runtime)
+        self.feed_forward_out_norm = None
+        if spec.feed_forward is not None:
+            self.feed_forward_out_norm = NORMS.build(spec.feed_forward_out_norm, runtime)
+
+    def children(self):
+        out = super().children()
+        out[self.spec.mixer_out_norm_name] = self.mixer_out_norm
+        if self.feed_forward is not None:
+            out[self.spec.feed_forward_out_norm_name] = self.feed_forward_out_norm
+        return out
+
+    def _join(self, residual, y, out_norm, next_norm):
+        """residual += out_norm(y); the rows of ``next_norm`` over the sum, or None."""
+        form = getattr(out_norm, "row_and_column_form", None)
+        next_form = getattr(next_norm, "row_and_column_form", None)
+        if form is None:
+            K.add_into(residual, out_norm.forward(y))
+            return None if next_norm is None else next_norm.forward(residual)
+        weight, eps = form()
+        if next_form is None:
+            K.normed_add(residual, y, weight, eps)
+            return None if next_norm is None else next_norm.forward(residual)
+        next_weight, next_eps = next_form()
+        return K.normed_add(residual, y, weight, eps, next_weight, next_eps, self.rt.dtype)
+
+    def forward(self, residual, batch, entry):
+        if isinstance(residual, ResidualStream):
+            residual = residual.tensor
+        x = self.mixer_norm.forward(residual)
+        y = torch.zeros_like(residual)
+        self.mixer.forward(x, batch, entry, y)
+        h = self._join(residual, y, self.mixer_out_norm, self.feed_forward_norm)
+        if self.feed_forward is not None:
+            y.zero_()
+            self.feed_forward.forward(h, batch, y)
+            self._join(residual, y, self.feed_forward_out_norm, None)
+
+
 register_block("pre_norm", PreNormBlock)
+register_block("sandwich_norm", SandwichNormBlock)

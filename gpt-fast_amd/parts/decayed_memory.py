@@ -1,0 +1,74 @@
+"""Linear attention with a fixed decay per head (lightning attention)."""
+import dataclasses
+
+import torch
+
+from ..cache.store import StateNeed
+from ..config.spec import DecayedMemorySpec
+from ..ops import decayed_memory as M
+from ..ops import linear as L
+from .base import Param, Part, Runtime, add_late, check_bound, register_mixer
+
+
+class DecayedMemory(Part):
+    """Per head a state ``S [dk, dv]``, float32, zero at a sequence's start, kept in the
+    cache's state slot of the sequence and carried from step to step:
+
+        q = silu(w_q x)   k = silu(w_k x)   v = silu(w_v x)
+        S' = decay_h S + k v^T          o = S'^T q
+
+    then the heads' results side by side over their root mean square, times ``norm``, times
+    sigmoid(w_g x), then ``wo``.  The four input projections are one matrix ``w_in`` (rows of
+    q, k, v, g) whose product keeps its float32 sums: the activations, the state and
+    everything up to the operand of ``wo`` are float32 whatever the engine's type."""
+
+    replayable = True
+    libraries = ("decayed_memory",)
+    defers_sum = True              # ``residual`` may be a parts.base.ResidualStream
+
+    def __init__(self, spec: DecayedMemorySpec, runtime: Runtime):
+        if spec.key_dim > M.MAX_KEY_DIM:
+            raise ValueError(f"decayed memory: key_dim {spec.key_dim} > {M.MAX_KEY_DIM}")
+        if len(spec.decay) != spec.n_heads:
+            raise ValueError(f"decayed memory: {len(spec.decay)} decays for {spec.n_heads} heads")
+        self.spec = spec
+        self.rt = runtime
+        rows = M.RowLayout.fused(spec.n_heads, spec.key_dim, spec.value_dim)
+        self.in_rows = rows.width                       # rows of w_in as it is stored
+        self.rows = dataclasses.replace(rows, width=(rows.width + 7) // 8 * 8)
+        self.decay = torch.tensor(spec.decay, dtype=torch.float64).to(torch.float32).to(runtime.device)
+        self.w_in = self.wo = self.norm = None
+
+    def parameters(self):
+        s = self.spec
+        return {"w_in": Param((self.in_rows, s.dim)),
+                "norm": Param((s.n_heads * s.value_dim,), role="vector", init="norm"),
+                "wo": Param((s.dim, s.n_heads * s.value_dim))}
+
+    def bind(self, tensors):
+        check_bound("DecayedMemory", self.parameters(), tensors)
+        # zero rows up to a multiple of eight: the products' kernels store whole groups
+        self.w_in, self.wo = L.pad_rows(tensors["w_in"], 8), tensors["wo"]
+        self.norm = tensors["norm"].to(torch.float32).contiguous()
+
+    def cache_need(self):
+        s = self.spec
+        return StateNeed((M.state_size(s.n_heads, s.key_dim, s.value_dim),), "float32")
+
+    def step_flops(self, q_lens, starts) -> float:
+        s = self.spec
+        n = sum(q_lens)
+        cell = 2.0 * 2.0 * s.n_heads * s.key_dim * s.value_dim          # update and read of S
+        return n * (2.0 * (self.in_rows + s.n_heads * s.value_dim) * s.dim + cell)
+
+    def forward(self, x, batch, entry, residual):
+        s = self.spec
+        proj = L.linear(x, self.w_in, out_dtype=torch.float32)
+        o = M.cell(proj, self.rows, self.decay, entry.state, batch.q_start, batch.slots,
+                   batch.n_seqs, batch.max_q_len, s.n_heads, s.key_dim, s.value_dim)
+        y = M.row_norm_gate(o, self.norm, proj, self.rows, s.eps, self.rt.dtype)
+        add_late(residual, lambda rows, then_norm, takes_halves: L.linear_into(
+            y, self.wo, rows, then_norm, takes_halves))
+
+
+register_mixer("decayed_memory", DecayedMemory)

@@ -1,5 +1,10 @@
 """Gated feed-forward (reference model.py:219-227)."""
-from ..config.spec import GatedFeedForwardSpec
+import math
+
+import torch
+
+from ..config.spec import DenseFeedForwardSpec, GatedFeedForwardSpec
+from ..ops import kernels as K
 from ..ops import linear as L
 from .base import Param, Part, Runtime, add_late, check_bound, register_feed_forward
 
@@ -42,3 +47,52 @@ class GatedFeedForward(Part):
 
 
 register_feed_forward("gated", GatedFeedForward)
+
+
+def _softplus(z: float) -> float:
+    return max(z, 0.0) + math.log1p(math.exp(-abs(z)))
+
+
+class DenseFeedForward(Part):
+    """``w_down( act(w_up x) )`` without biases and without a gate.  ``activation`` "xielu"
+    has two learned numbers p, q (the parameter ``act``): for z > 0 ``softplus(p) z^2 + z/2``,
+    for z <= 0 ``(1/2 + softplus(q)) (exp(z) - 1 - z) + z/2``; the two factors are worked out
+    once, when the weights are bound.  "silu" and "gelu_tanh" have no parameter."""
+
+    replayable = True
+    defers_sum = True              # ``residual`` may be a parts.base.ResidualStream
+
+    def __init__(self, spec: DenseFeedForwardSpec, runtime: Runtime):
+        if spec.activation not in K.ACTIVATIONS:
+            raise ValueError(f"activation '{spec.activation}': {sorted(K.ACTIVATIONS)}")
+        self.spec = spec
+        self.rt = runtime
+        self.w_up = self.w_down = None
+        self.a = self.b = 0.0
+
+    def parameters(self):
+        s = self.spec
+        p = {"w_up": Param((s.hidden, s.dim)), "w_down": Param((s.dim, s.hidden))}
+        if s.activation == "xielu":
+            p["act"] = Param((2,), role="vector", init="unit")
+        return p
+
+    def bind(self, tensors):
+        check_bound("DenseFeedForward", self.parameters(), tensors)
+        self.w_up, self.w_down = tensors["w_up"], tensors["w_down"]
+        if self.spec.activation == "xielu":
+            p, q = (float(v) for v in tensors["act"].to(torch.float32).cpu())
+            self.a, self.b = _softplus(p), 0.5 + _softplus(q)
+
+    def step_flops(self, q_lens, starts) -> float:
+        return 2.0 * sum(q_lens) * 2 * self.spec.hidden * self.spec.dim
+
+    def forward(self, x, batch, residual):
+        def finish(rows, then_norm, takes_halves):
+            h = L.linear(x, self.w_up)
+            K.activate(h, self.spec.activation, self.a, self.b, out=h)
+            return L.linear_into(h, self.w_down, rows, then_norm, takes_halves)
+        add_late(residual, finish)
+
+
+register_feed_forward("dense", DenseFeedForward)

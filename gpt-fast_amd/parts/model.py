@@ -6,7 +6,8 @@ import torch
 from ..config.spec import ModelPlan
 from ..ops import kernels as K
 from ..ops import linear as L
-from .base import BLOCKS, NORMS, POSITIONS, Param, ResidualStream, Runtime, check_bound
+from .base import (BLOCKS, NORMS, POSITIONS, STREAM_STEPS, Param, ResidualStream, Runtime,
+                   check_bound)
 
 
 class DecoderModel:
@@ -31,7 +32,17 @@ class DecoderModel:
             if not hasattr(self.input_position, "add_to_stream"):
                 raise TypeError(f"position kind '{plan.input_position.kind}' cannot be a plan's "
                                 f"input_position: its part has no add_to_stream(residual, batch)")
+        # steps on the stream that stand before a run (Run.enter), one part per spec: runs that
+        # name the same spec share its parameters
+        self.enter_steps = {}
+        for run in plan.order:
+            spec = getattr(run, "enter", None)
+            if spec is not None and spec not in self.enter_steps:
+                self.enter_steps[spec] = STREAM_STEPS.build(spec, runtime)
         self.embedding = self.head = None
+        # ``tap(n, rows)`` is called with the float32 stream [N, D] after run n of the order
+        # (tracing, tests); None: nothing is called
+        self.tap = None
 
     # ------------------------------------------------------------------ parameters
     def parameters(self) -> Dict[str, Param]:
@@ -42,6 +53,8 @@ class DecoderModel:
         if self.input_position is not None:
             for name, param in self.input_position.parameters().items():
                 p[f"{self.plan.input_position_name}.{name}"] = param
+        for step in self.enter_steps.values():
+            p.update(step.parameters())             # under their own full names
         for layer, block in zip(self.plan.layers, self.blocks):
             for name, param in block.parameters().items():
                 p[f"{layer.name}.{name}"] = param
@@ -62,6 +75,8 @@ class DecoderModel:
             prefix = self.plan.input_position_name + "."
             self.input_position.bind({k[len(prefix):]: v for k, v in tensors.items()
                                       if k.startswith(prefix)})
+        for step in self.enter_steps.values():
+            step.bind({k: tensors[k] for k in step.parameters()})
         for layer, block in zip(self.plan.layers, self.blocks):
             prefix = layer.name + "."
             block.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
@@ -84,6 +99,7 @@ class DecoderModel:
         """Every part issues the same kernels whatever a batch holds: a recorded step can be
         replayed."""
         return (all(getattr(b, "replayable", False) for b in self.blocks)
+                and all(getattr(s, "replayable", False) for s in self.enter_steps.values())
                 and getattr(self.final_norm, "replayable", False)
                 and (self.input_position is None
                      or getattr(self.input_position, "replayable", False)))
@@ -116,6 +132,9 @@ class DecoderModel:
         for run in self.plan.order:
             block = self.blocks[run.layer]
             flops += getattr(block, "step_flops", lambda q, s: 0.0)(q_lens, starts)
+            if getattr(run, "enter", None) is not None:
+                flops += getattr(self.enter_steps[run.enter], "step_flops",
+                                 lambda q, s: 0.0)(q_lens, starts)
         return flops
 
     def kernel_libraries(self):
@@ -133,7 +152,8 @@ class DecoderModel:
                     names.append(n)
             for child in getattr(part, "children", lambda: {})().values():
                 visit(child)
-        for part in list(self.blocks) + [self.final_norm, self.input_position]:
+        for part in list(self.blocks) + list(self.enter_steps.values()) \
+                + [self.final_norm, self.input_position]:
             if part is not None:
                 visit(part)
         return names
@@ -158,10 +178,21 @@ class DecoderModel:
         if self.input_position is not None:
             self.input_position.add_to_stream(residual, batch)
         stream = ResidualStream(residual)
+        # the embedded rows, for steps that mix them into the stream again; a copy where a
+        # block may have changed the stream (in place) before the first such step
+        embedded = None
+        if self.enter_steps:
+            embedded = residual if getattr(plan.order[0], "enter", None) is not None \
+                else residual.clone()
         for n, run in enumerate(plan.order):                              # model.py:142-143
+            if getattr(run, "enter", None) is not None:
+                stream = ResidualStream(self.enter_steps[run.enter].forward(
+                    stream.tensor, embedded, batch))
             block = self.blocks[run.layer]
             block.forward(stream if getattr(block, "takes_stream", False) else stream.tensor,
                           batch, cache.entries[n])
+            if self.tap is not None:
+                self.tap(n, stream.tensor)
         if batch.n_want == 0:
             stream.tensor
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32,
