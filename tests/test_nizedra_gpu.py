@@ -1,0 +1,595 @@
+"""Nizedra on the GPU against the plain float64 implementation of tests/plain_nizedra.py:
+each mechanism's kernels alone, whole prompts with the stream after every run, prompts in
+portions, token-by-token decoding, unequal batches, slots and pages that come back, a
+window's edge and far keys with inputs that make one key stand out, long memory, and greedy
+generation through the library's generation loop, command line and trace replay."""
+import math
+
+import pytest
+import torch
+
+import plain_nizedra as P
+import util
+from nizedra_cases import CASES, make_folder
+from util import TOL_BF16, TOL_F32, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+# The decayed memory sums a sequence chunk by chunk, the plain loop token by token in float64;
+# a float32 engine stays within this of it over a few hundred tokens.
+TOL_F32_LONG = 1e-4
+
+
+def row_errors(got, want):
+    """Per row: root mean square of the difference over that of all of ``want``."""
+    got, want = got.double().cpu(), want.double().cpu()
+    return (got - want).pow(2).mean(-1).sqrt() / want.pow(2).mean().sqrt()
+
+
+def bf16_close(got, want):
+    """A bfloat16 engine against float64.  Rows differ in how much they amplify a rounding
+    error: every sublayer's result is divided by its own root mean square before it joins the
+    stream, and a head of the decayed memory whose q . k nearly cancels at a sequence's first
+    token turns the rounding of its input into an error of a third of that row, which the
+    later tokens then read (seen with one of these tests' token sequences: the stream of the
+    float32 engine and of this one differ by 4 % before that sublayer and by 34 % in its
+    result at row 0).  So the typical row is held to the tolerance, and all but one in a
+    hundred (at least one) to a bound that a wrong key, a lost state or a missing term, which
+    touch most rows, would still break.  The float32 engine is the sharp test."""
+    e = row_errors(got, want).sort().values
+    rest = e[:max(1, e.numel() - max(1, e.numel() // 100))]
+    return float(rest.max()) < 0.3 and float(e.median()) < TOL_BF16
+
+
+def close(got, want, dtype, tol):
+    return bf16_close(got, want) if dtype == "bfloat16" else rel_err(got, want) < tol
+
+
+def _engine(folder, dtype, **kw):
+    import gpt_fast_amd as gfa
+    kw.setdefault("max_tokens", 4096)
+    return gfa.Engine.from_folder(folder, dtype=dtype, device=DEV, **kw)
+
+
+def _steps(eng, toks, cuts):
+    """Feed ``toks`` as one sequence in portions that end at ``cuts``; logits of every token."""
+    import gpt_fast_amd as gfa
+    slot = eng.start_sequence()
+    out, lo = [], 0
+    for hi in list(cuts) + [len(toks)]:
+        if hi <= lo:
+            continue
+        out.append(eng.step([gfa.Entry(slot, toks[lo:hi], want=list(range(hi - lo)))]).cpu())
+        lo = hi
+    eng.end_sequence(slot)
+    return torch.cat(out)
+
+
+# --------------------------------------------------------------------------- mechanisms alone
+def test_activation_kernel():
+    from gpt_fast_amd.ops import kernels as K
+    torch.manual_seed(0)
+    for p, q in ((0.7, -1.3), (0.0, 0.0), (-2.0, 3.0)):
+        a, b = P.softplus(p), 0.5 + P.softplus(q)
+        for dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 1e-2)):
+            for shape in ((19, 37), (5, 64)):
+                x = (torch.randn(*shape, device=DEV) * 3).to(dtype)
+                x[0, :3] = torch.tensor([0.0, -20.0, 20.0])
+                want = P.xielu(x.double().cpu(), p, q)
+                assert rel_err(K.activate(x, "xielu", a, b), want) < tol
+    x = torch.randn(7, 24, device=DEV) * 3
+    assert rel_err(K.activate(x, "silu"), torch.nn.functional.silu(x.double().cpu())) < 1e-6
+    z = x.double().cpu()
+    gelu = 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+    assert rel_err(K.activate(x, "gelu_tanh"), gelu) < 1e-6
+
+
+def test_a_result_joins_the_stream_through_its_norm():
+    from gpt_fast_amd.ops import kernels as K
+    torch.manual_seed(1)
+    for dim in (50, 96, 1030):
+        res = torch.randn(9, dim, device=DEV) * 2
+        y = torch.randn(9, dim, device=DEV) * 5
+        w1, w2 = torch.randn(dim, device=DEV), torch.randn(dim, device=DEV)
+        want = res.double().cpu() + P.rms_norm(y.double().cpu(), w1.double().cpu(), 1e-3)
+        want_next = P.rms_norm(want, w2.double().cpu(), 1e-6)
+        r1 = res.clone()
+        assert K.normed_add(r1, y, w1, 1e-3) is None
+        assert rel_err(r1, want) < 1e-6
+        for dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 1e-2)):
+            r2 = res.clone()
+            nxt = K.normed_add(r2, y, w1, 1e-3, w2, 1e-6, dtype)
+            assert torch.equal(r1, r2)
+            assert rel_err(nxt, want_next) < tol
+
+
+def test_rows_side_by_side_and_a_bias():
+    from gpt_fast_amd.ops import kernels as K
+    torch.manual_seed(2)
+    a, b = torch.randn(5, 34, device=DEV), torch.randn(5, 34, device=DEV)
+    assert torch.equal(K.concat_rows(a, b, torch.float32), torch.cat([a, b], 1))
+    assert torch.equal(K.concat_rows(a, b, torch.bfloat16), torch.cat([a, b], 1).bfloat16())
+    bias = torch.randn(34, device=DEV)
+    assert torch.equal(K.add_bias(a.clone(), bias), a + bias)
+
+
+def test_batched_float_product_with_strides():
+    from gpt_fast_amd.ops import kernels as K
+    torch.manual_seed(3)
+    a = torch.randn(3, 70, 20, device=DEV)
+    w = torch.randn(3, 20, 33, device=DEV).transpose(1, 2)          # [3, 33, 20] as a view
+    full = torch.zeros(3, 70, 40, device=DEV)
+    K.gemm_f32_batched(a, w, full[:, :, :33])
+    want = torch.einsum("bmk,bnk->bmn", a.double().cpu(), w.double().cpu())
+    assert rel_err(full[:, :, :33], want) < 1e-6
+    assert float(full[:, :, 33:].abs().max()) == 0.0
+    y = torch.zeros(70, 3, 33, device=DEV)                          # rows token by token
+    K.gemm_f32_batched(a, w, y.permute(1, 0, 2))
+    assert rel_err(y.permute(1, 0, 2), want) < 1e-6
+
+
+def test_distance_rows_of_the_bias_table():
+    from gpt_fast_amd.ops.scored_attention import distance_rows
+    for rows, far in ((8, 50), (6, 9), (32, 2000), (7, 300), (5, 11), (16, 128)):
+        table = distance_rows(rows, far)
+        for n in range(len(table)):
+            assert table[n] == P.distance_bucket(n, rows, far), (rows, far, n)
+        assert table[-1] == rows - 1 and P.distance_bucket(10 * int(far), rows, far) == rows - 1
+        assert table[:rows // 2] == list(range(rows // 2))
+        assert all(x <= y for x, y in zip(table, table[1:]))
+
+
+@pytest.mark.parametrize("H,dk,dv", [(2, 16, 32), (1, 24, 40), (3, 20, 12), (2, 72, 8), (1, 130, 33),
+                                     (3, 10, 6), (2, 128, 128), (2, 64, 16)])
+@pytest.mark.parametrize("chunked", [False, True])
+def test_decayed_memory_kernels_alone(H, dk, dv, chunked):
+    """Three sequences of unequal length in one launch, then a second launch that goes on
+    from the state the first one left, in other slots than their order."""
+    from gpt_fast_amd.ops import decayed_memory as M
+    torch.manual_seed(H * 100 + dk)
+    if chunked and not M.chunks_available(dk, dv):
+        pytest.skip("the chunked kernel does not take these sizes")
+    rows = M.RowLayout.fused(H, dk, dv)
+    lens1, lens2 = ([5, 1, 37], [1, 9, 2]) if not chunked else ([5, 64, 137], [64, 9, 133])
+    slots = [4, 0, 2]
+    state = torch.zeros(6, M.state_size(H, dk, dv), device=DEV)
+    state[1].fill_(7.0)                                        # a slot nobody uses stays as it is
+    decay = torch.tensor([0.999, 0.6, 0.93][:H], device=DEV)
+    weight = 1 + 0.2 * torch.randn(H * dv, device=DEV)
+    seqs = [torch.randn(a + b, rows.width, device=DEV) * 1.5 for a, b in zip(lens1, lens2)]
+    got = [[] for _ in seqs]
+    for part, lens in ((0, lens1), (1, lens2)):
+        chunks = [s[:l] if part == 0 else s[-l:] for s, l in zip(seqs, lens)]
+        proj = torch.cat(chunks).contiguous()
+        q_start = torch.tensor([sum(lens[:b]) for b in range(len(lens) + 1)], dtype=torch.int32, device=DEV)
+        o = M.scan(proj, rows, decay, state, q_start, torch.tensor(slots, dtype=torch.int32, device=DEV),
+                   3, H, dk, dv, chunked=chunked)
+        y = M.row_norm_gate(o, weight, proj, rows, 1e-5, torch.float32)
+        at = 0
+        for b, l in enumerate(lens):
+            got[b].append(y[at:at + l].double().cpu())
+            at += l
+    assert torch.all(state[1] == 7.0)
+    silu = torch.nn.functional.silu
+    for b, s in enumerate(seqs):
+        p = s.double().cpu()
+        T = p.shape[0]
+        q = silu(p[:, rows.q:rows.k]).view(T, H, dk)
+        k = silu(p[:, rows.k:rows.v]).view(T, H, dk)
+        v = silu(p[:, rows.v:rows.g]).view(T, H, dv)
+        o, S = P.decayed_memory_cell(q, k, v, decay.double().cpu())
+        want = (P.rms_norm(o.reshape(T, H * dv), weight.double().cpu(), 1e-5)
+                * torch.sigmoid(p[:, rows.g:rows.g + H * dv]))
+        assert rel_err(torch.cat(got[b]), want) < 2e-5
+        assert rel_err(state[slots[b]].double().cpu().view(H, dk, dv), S) < 2e-5
+
+
+def _plain_scored_attention(q, k, v, start, scale, window, temp, cap, bias, far, talk):
+    """q [T, H, d] are the last T of the sequence's tokens; k [L, G, d], v [L, G, dv]."""
+    T, H, _ = q.shape
+    L, G, _ = k.shape
+    s = torch.empty(H, T, L, dtype=torch.float64)
+    for h in range(H):
+        z = (q[:, h] @ k[:, h // (H // G)].T) * scale
+        if temp is not None:
+            z = z * temp[h]
+        if cap:
+            z = cap * torch.tanh(z / cap)
+        if bias is not None:
+            rows = bias.shape[0]
+            dist = torch.tensor([[P.distance_bucket(start + i - j, rows, far) if j <= start + i else 0
+                                  for j in range(L)] for i in range(T)])
+            z = z + bias[dist, h]
+        s[h] = z
+    if talk is not None:
+        s = torch.einsum("hg,gij->hij", talk, s)
+    i = torch.arange(T)[:, None] + start
+    j = torch.arange(L)[None, :]
+    see = (j <= i) if not window else (j <= i) & (i - j < window)
+    a = torch.softmax(s.masked_fill(~see, -math.inf), -1)
+    return torch.stack([a[h] @ v[:, h // (H // G)] for h in range(H)], 1)        # [T, H, dv]
+
+
+def _scored_attention_alone(dtype, H, G, d, dv, window, lens, starts, mixed, head_major=False,
+                            boost=None, cap=7.0, far=40.0, rows=8):
+    """The attention kernel over sequences that already hold ``starts[b]`` tokens and get
+    ``lens[b]`` more, pages handed out in reverse, against the plain attention.  ``boost``:
+    (sequence, key position, factor) multiplies that key, so that its score stands out."""
+    from gpt_fast_amd.ops import scored_attention as SA
+    torch.manual_seed(d * 7 + dv + H)
+    total = [s + l for s, l in zip(starts, lens)]
+    n_pages = sum((t + 63) // 64 for t in total)
+    order = list(range(n_pages))[::-1]
+    tables, at = [], 0
+    for t in total:
+        n = (t + 63) // 64
+        tables.append(order[at:at + n])
+        at += n
+    widest = max(len(t) for t in tables)
+    table = torch.tensor([t + [-1] * (widest - len(t)) for t in tables], dtype=torch.int32, device=DEV)
+    ks = [(torch.randn(t, G, d) * 1.0).to(dtype) for t in total]
+    vs = [torch.randn(t, G, dv).to(dtype) for t in total]
+    qs = [torch.randn(l, H, d).to(dtype) for l in lens]
+    if boost is not None:
+        b, key, factor = boost
+        ks[b][key] *= factor
+    # pages as keys [n, G, 64, d] and values [n, G, dv, 64]; what lies beyond a sequence's end is
+    # not a number: a kernel that reads it spoils its sums
+    k_rows = torch.full((n_pages, G, 64, d), float("nan"), dtype=dtype)
+    v_cols = torch.full((n_pages, G, dv, 64), float("nan"), dtype=dtype)
+    for b, t in enumerate(total):
+        for pos in range(t):
+            page = tables[b][pos // 64]
+            k_rows[page, :, pos % 64] = ks[b][pos]
+            v_cols[page, :, :, pos % 64] = vs[b][pos]
+    k_pages = torch.empty_like(k_rows).view(n_pages, G, -1)
+    v_pages = torch.empty_like(v_cols).view(n_pages, G, -1)
+    k_pages[..., util.key_places(d).reshape(-1)] = k_rows.reshape(n_pages, G, -1)
+    v_pages[..., util.value_places(dv).reshape(-1)] = v_cols.reshape(n_pages, G, -1)
+    k_pages, v_pages = k_pages.view_as(k_rows).to(DEV), v_pages.view_as(v_cols).to(DEV)
+    temp = (1 + 0.3 * torch.randn(H)) if mixed else None
+    bias = torch.randn(rows, H) * 2 if mixed else None
+    talk = (torch.eye(H) + 0.3 * torch.randn(H, H)) if mixed else None
+    lookup = torch.tensor(SA.distance_rows(rows, far), dtype=torch.int32, device=DEV) if mixed else None
+    q = torch.cat(qs).to(DEV)
+    tok_seq = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)
+    tok_pos = torch.tensor([s + i for s, l in zip(starts, lens) for i in range(l)], dtype=torch.int32, device=DEV)
+    dev = lambda t: None if t is None else t.float().to(DEV)
+    q_in = q.permute(1, 0, 2).contiguous() if head_major else q
+    out = SA.attention(q_in, k_pages, v_pages, tok_seq, tok_pos, table, 0.4, window=window or 0,
+                       temperature=dev(temp), softcap=cap if mixed else 0.0, bias=dev(bias),
+                       lookup=lookup, talk=dev(talk), head_major=head_major)
+    if head_major:
+        out = out.permute(1, 0, 2)
+    at, worst = 0, 0.0
+    dbl = lambda t: None if t is None else t.double()
+    for b, l in enumerate(lens):
+        want = _plain_scored_attention(qs[b].double(), ks[b].double(), vs[b].double(), starts[b], 0.4,
+                                       window, dbl(temp), cap if mixed else None, dbl(bias), far, dbl(talk))
+        got = out[at:at + l].double().cpu()
+        assert not torch.isnan(got).any()
+        worst = max(worst, rel_err(got, want))
+        at += l
+    return worst
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("H,G,d,dv,window,mixed,head_major", [
+    (4, 2, 16, 16, None, True, False), (3, 3, 20, 12, None, True, False), (6, 1, 8, 24, None, True, False),
+    (2, 1, 10, 6, None, True, False), (16, 4, 32, 64, None, True, False), (20, 5, 16, 48, None, True, False),
+    (3, 1, 40, 32, 24, False, True), (2, 1, 28, 20, None, False, True), (4, 1, 160, 144, 70, False, True),
+    (2, 1, 16, 10, 9, False, True), (5, 1, 576, 512, 100, False, True), (4, 2, 64, 64, 33, False, False)])
+def test_scored_attention_alone(dtype, tol, H, G, d, dv, window, mixed, head_major):
+    """A prompt, a portion at an offset, single tokens and a first token, in one launch."""
+    err = _scored_attention_alone(dtype, H, G, d, dv, window, lens=[130, 40, 1, 1, 3], starts=[0, 70, 200, 0, 63],
+                                  mixed=mixed, head_major=head_major)
+    assert err < tol
+
+
+@pytest.mark.parametrize("window", [24, 64, 100])
+@pytest.mark.parametrize("offset", [0, 1])
+def test_a_key_at_the_windows_edge_stands_out(window, offset):
+    """One key is multiplied by 30: with it just inside the window of the last token it takes
+    the softmax, just outside it must not be seen, in a prompt and in a single-token step."""
+    for lens, starts in (([200], [0]), ([1], [199])):
+        key = 199 - window + 1 - offset                 # offset 0: the last key seen; 1: the first not
+        err = _scored_attention_alone(torch.float32, 3, 1, 40, 32, window, lens, starts, mixed=False,
+                                      head_major=True, boost=(0, key, 30.0))
+        assert err < 2e-5
+
+
+@pytest.mark.parametrize("key", [0, 1, 63, 64, 65, 127, 128, 300, 449])
+def test_a_far_key_among_hundreds_stands_out(key):
+    """No window: one key far back, at a page's border, the first, the last, takes the softmax;
+    the bias of the far distances and the mix across heads apply to it."""
+    for lens, starts in (([450], [0]), ([2], [448])):
+        err = _scored_attention_alone(torch.float32, 4, 2, 16, 16, None, lens, starts, mixed=True,
+                                      boost=(0, key, 12.0), cap=50.0, far=300.0, rows=12)
+        assert err < 2e-5
+
+
+# --------------------------------------------------------------------------- whole models
+@pytest.mark.parametrize("name", sorted(CASES))
+@pytest.mark.parametrize("dtype,tol", [("float32", TOL_F32_LONG), ("bfloat16", TOL_BF16)])
+def test_whole_prompt_at_every_position_and_the_stream_after_every_run(tmp_path, name, dtype, tol):
+    folder = make_folder(tmp_path, name, seed=11)
+    cfg, w = P.load_folder(folder)
+    toks = util.random_tokens(cfg["vocab"], 150, 3)
+    outs = []
+    want = P.forward(w, cfg, toks, outs)
+    eng = _engine(folder, dtype)
+    taps = []
+    eng.model.tap = lambda n, x: taps.append(x.double().cpu())
+    got = _steps(eng, toks, [])
+    eng.model.tap = None
+    assert close(got, want, dtype, tol)
+    assert len(taps) == len(outs) == len(P.run_order(cfg))
+    if dtype == "float32":
+        for n, (a, b) in enumerate(zip(taps, outs)):
+            assert rel_err(a, b) < TOL_F32_LONG, n
+        # one token, and the first tokens of a sequence
+        assert rel_err(_steps(eng, toks[:1], []), want[:1]) < TOL_F32
+        assert rel_err(_steps(eng, toks[:3], []), want[:3]) < TOL_F32
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C", "O"])
+@pytest.mark.parametrize("dtype,tol", [("float32", TOL_F32_LONG), ("bfloat16", TOL_BF16)])
+def test_portions_and_token_by_token_equal_the_whole_prompt(tmp_path, name, dtype, tol):
+    folder = make_folder(tmp_path, name, seed=12)
+    cfg, w = P.load_folder(folder)
+    toks = util.random_tokens(cfg["vocab"], 210, 5)
+    want = P.forward(w, cfg, toks)
+    eng = _engine(folder, dtype)
+    whole = _steps(eng, toks, [])
+    assert close(whole, want, dtype, tol)
+    for cuts in ([2, 4, 5, 70, 128, 129], [63, 64, 65, 192], [17, 150], list(range(150, 210)),
+                 list(range(1, 80))):
+        got = _steps(eng, toks, cuts)
+        assert close(got, want, dtype, tol), cuts
+        assert close(got, whole, dtype, tol), cuts
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("dtype,same", [("float32", 2e-5), ("bfloat16", TOL_BF16)])
+def test_unequal_batches_equal_each_request_alone(tmp_path, name, dtype, same):
+    import gpt_fast_amd as gfa
+    folder = make_folder(tmp_path, name, seed=13)
+    cfg, w = P.load_folder(folder)
+    lens = [1, 5, 131, 64, 70]
+    tail = 30
+    seqs = [util.random_tokens(cfg["vocab"], n + tail, 40 + n) for n in lens]
+    eng = _engine(folder, dtype, max_tokens=64 * 20, max_sequences=6)
+    alone = [_steps(eng, s, [n] + list(range(n + 1, n + tail))) for s, n in zip(seqs, lens)]
+    slots = [eng.start_sequence() for _ in seqs]
+    got = [[] for _ in seqs]
+    out = eng.step([gfa.Entry(sl, s[:n], want=list(range(n))) for sl, s, n in zip(slots, seqs, lens)]).cpu()
+    at = 0
+    for b, n in enumerate(lens):
+        got[b].append(out[at:at + n])
+        at += n
+    live = list(range(len(seqs)))
+    for t in range(tail):
+        if t == 10:                                  # a shorter request ends earlier
+            eng.end_sequence(slots[1])
+            live.remove(1)
+        out = eng.step([gfa.Entry(slots[b], [seqs[b][lens[b] + t]], want=[0]) for b in live]).cpu()
+        for i, b in enumerate(live):
+            got[b].append(out[i:i + 1])
+    for b in live:
+        eng.end_sequence(slots[b])
+    eng.cache.check()
+    for b, s in enumerate(seqs):
+        g = torch.cat(got[b])
+        assert close(g, alone[b][:g.shape[0]], dtype, same), b
+    want = P.forward(w, cfg, seqs[2])
+    assert close(torch.cat(got[2]), want, dtype, TOL_F32_LONG)
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_step_that_mixes_single_tokens_a_portion_and_a_new_prompt(tmp_path, name, dtype):
+    import gpt_fast_amd as gfa
+    folder = make_folder(tmp_path, name, seed=21)
+    cfg, w = P.load_folder(folder)
+    _, before, mixed = util.mixed_step_case(cfg["vocab"])
+    lens = {"d0": 9, "d1": 66, "d2": 130, "c": 112, "p": 131}
+    # token sequences that the plain implementation, with its norms' results rounded to
+    # bfloat16, follows within a few percent (some sequences amplify that rounding tenfold)
+    seqs = {r: util.random_tokens(cfg["vocab"], n, 300 + n) for r, n in lens.items()}
+    eng = _engine(folder, dtype, max_tokens=64 * 16, max_sequences=5)
+    slots = {r: eng.start_sequence() for r in seqs}
+    got = {r: [] for r in seqs}
+    order = ["d0", "d1", "d2", "c"]
+    logits = eng.step([gfa.Entry(slots[r], seqs[r][:before[r]], want=list(range(before[r]))) for r in order]).cpu()
+    at = 0
+    for r in order:
+        got[r].append(logits[at:at + before[r]])
+        at += before[r]
+    order = ["d0", "c", "d1", "p", "d2"]
+    fed = {r: before.get(r, 0) for r in order}
+    logits = eng.step([gfa.Entry(slots[r], seqs[r][fed[r]:fed[r] + mixed[r]], want=list(range(mixed[r])))
+                       for r in order]).cpu()
+    at = 0
+    for r in order:
+        got[r].append(logits[at:at + mixed[r]])
+        at += mixed[r]
+        fed[r] += mixed[r]
+    for r in ("c", "p"):
+        while fed[r] < len(seqs[r]):
+            got[r].append(eng.step([gfa.Entry(slots[r], [seqs[r][fed[r]]], want=[0])]).cpu())
+            fed[r] += 1
+    for r, toks in seqs.items():
+        assert close(torch.cat(got[r]), P.forward(w, cfg, toks), dtype, TOL_F32_LONG), r
+        eng.end_sequence(slots[r])
+    eng.cache.check()
+    assert eng.cache.slots.held == 0
+
+
+def test_slots_and_pages_that_come_back_start_clean(tmp_path):
+    """A cache of few pages and two slots: requests follow one another in the same slots and
+    pages, long decoding gives the window's pages back, and every request equals the plain
+    computation of itself alone."""
+    import gpt_fast_amd as gfa
+    folder = make_folder(tmp_path, "A", seed=14)
+    cfg, w = P.load_folder(folder)
+    eng = _engine(folder, "float32", max_tokens=64 * 7, max_sequences=2)
+    for round_ in range(3):
+        a = util.random_tokens(cfg["vocab"], 150 + 90, 60 + round_)
+        b = util.random_tokens(cfg["vocab"], 40 + 90, 70 + round_)
+        sa, sb = eng.start_sequence(), eng.start_sequence()
+        assert {sa, sb} == {0, 1}
+        got_a, got_b = [], []
+        out = eng.step([gfa.Entry(sa, a[:150], want=[149]), gfa.Entry(sb, b[:40], want=[39])]).cpu()
+        got_a.append(out[0:1])
+        got_b.append(out[1:2])
+        for t in range(89):
+            out = eng.step([gfa.Entry(sa, [a[150 + t]], want=[0]), gfa.Entry(sb, [b[40 + t]], want=[0])]).cpu()
+            got_a.append(out[0:1])
+            got_b.append(out[1:2])
+        eng.cache.check()
+        eng.end_sequence(sb)
+        eng.end_sequence(sa)
+        assert rel_err(torch.cat(got_a), P.forward(w, cfg, a[:-1])[149:]) < TOL_F32_LONG
+        assert rel_err(torch.cat(got_b), P.forward(w, cfg, b[:-1])[39:]) < TOL_F32_LONG
+    for _, g in eng.cache.kv_groups:
+        assert g.pages.held == 0
+
+
+def test_a_memory_written_far_back_is_read_hundreds_of_tokens_later(tmp_path):
+    """Decays close to one: what the states hold after 500 tokens comes from all of them.
+    Decoding the last 40 alone reads it through the carried state of every pass of the loop; a
+    state that was lost, reset or shared between passes would show."""
+    config = {**CASES["A"], "layers": [dict(l) for l in CASES["A"]["layers"]]}
+    for l in config["layers"]:
+        if l["type"] == "lightning":
+            l["mixer"] = {**l["mixer"], "decay": [0.9995] * l["mixer"]["heads"]}
+    from nizedra_cases import write_model
+    folder = write_model(str(tmp_path / "far"), config, 15)
+    cfg, w = P.load_folder(folder)
+    toks = util.random_tokens(cfg["vocab"], 540, 9)
+    want = P.forward(w, cfg, toks)
+    # it matters: the same tokens without the first 300 give other logits at the end
+    assert rel_err(P.forward(w, cfg, toks[300:])[-40:], want[-40:]) > 1e-2
+    for dtype, tol in (("float32", TOL_F32_LONG), ("bfloat16", TOL_BF16)):
+        eng = _engine(folder, dtype)
+        got = _steps(eng, toks, [500] + list(range(501, 540)))
+        assert close(got[-41:], want[-41:], dtype, tol)
+        assert close(got, want, dtype, tol)
+
+
+def test_peaked_softmax_over_a_long_prompt_and_decoding_past_the_window(tmp_path):
+    """Queries scaled up until a head's weight sits on one or two keys, among some hundred
+    candidates or at the window's edge; then 130 tokens decoded one by one, so that the
+    windows (24 and 70) pass over decoded tokens and pages are given back."""
+    def patch(t):
+        for name in t:
+            if name.endswith("mix.uq") or name.endswith("mix.temp"):
+                t[name] = t[name] * 5
+    for name in ("A", "C"):
+        folder = make_folder(tmp_path, name, seed=16, patch=patch, tag="peaked")
+        cfg, w = P.load_folder(folder)
+        toks = util.random_tokens(cfg["vocab"], 400, 21)
+        want = P.forward(w, cfg, toks)
+        for dtype in ("float32", "bfloat16"):
+            eng = _engine(folder, dtype, max_tokens=64 * 8, max_sequences=1)
+            got = _steps(eng, toks, [270] + list(range(271, 400)))
+            if dtype == "float32":
+                assert rel_err(got, want) < TOL_F32_LONG
+            else:
+                # scores five times as large carry five times the rounding of q and k into the
+                # softmax: bfloat16 is held to the typical row only
+                assert float(row_errors(got, want).median()) < TOL_BF16
+            eng.cache.check()
+
+
+# --------------------------------------------------------------------------- generation
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_greedy_generation_through_the_loop_and_the_recorded_step(tmp_path, name):
+    from gpt_fast_amd.engine.generate import generate
+    folder = make_folder(tmp_path, name, seed=17)
+    cfg, w = P.load_folder(folder)
+    prompts = [util.random_tokens(cfg["vocab"], n, 80 + n) for n in (7, 1, 90, 30)]
+    want = [P.greedy_generate(w, cfg, p, 12) for p in prompts]
+    eng = _engine(folder, "float32", max_tokens=64 * 12, max_sequences=4)
+    assert eng.model.replayable
+    for use_graph in (False, True, True):                       # the recording is replayed
+        got = generate(eng, prompts, max_new_tokens=12, temperature=0.0, use_graph=use_graph)
+        assert got.tokens == want, use_graph
+    # two at a time: slots and state come back between the batches
+    got = generate(eng, prompts, max_new_tokens=12, temperature=0.0, batch_size=2)
+    assert got.tokens == want
+    eng.cache.check()
+    # bfloat16 through the recorded step: the tokens of the step that is not recorded
+    eng = _engine(folder, "bfloat16", max_tokens=64 * 12, max_sequences=4)
+    plain_steps = generate(eng, prompts, max_new_tokens=12, temperature=0.0, use_graph=False).tokens
+    for _ in range(2):
+        assert generate(eng, prompts, max_new_tokens=12, temperature=0.0, use_graph=True).tokens == plain_steps
+
+
+def test_command_line_entry_point(tmp_path):
+    import gpt_fast_amd as gfa
+    folder = make_folder(tmp_path, "B", seed=18)
+    cfg, w = P.load_folder(folder)
+    prompt = util.random_tokens(cfg["vocab"], 20, 1)
+    lines = []
+    res = gfa.main(prompt=prompt, num_samples=1, max_new_tokens=8, temperature=0.0, top_k=None,
+                   checkpoint_path=folder, dtype="float32", device=DEV, out=lines.append)
+    assert res["result"].tokens[0] == P.greedy_generate(w, cfg, prompt, 8)
+    assert any("tokens/sec" in str(l) for l in lines)
+
+
+def test_trace_replay_program(tmp_path):
+    """bin/trace_run as a program on a Nizedra folder: two batches of unequal requests one after
+    the other (the second takes the slots, state and pages the first gave back), logits wanted
+    at some places only, steps in which nothing is wanted, a request that ends in the step that
+    brings its prompt."""
+    import json
+    import os
+    import subprocess
+
+    import numpy as np
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = make_folder(tmp_path, "A", seed=19)
+    cfg, w = P.load_folder(folder)
+    V = cfg["vocab"]
+    reqs = {"a": util.random_tokens(V, 150, 1), "b": util.random_tokens(V, 9, 2), "c": util.random_tokens(V, 1, 3),
+            "d": util.random_tokens(V, 200, 4), "e": util.random_tokens(V, 70, 5)}
+    prompt = {"a": 120, "b": 3, "c": 1, "d": 130, "e": 64}
+    steps, where = [], {r: [] for r in reqs}          # request -> (step, row in the file, position)
+    n = 0
+    for ids in (["a", "b", "c"], ["d", "e"]):
+        live, t = list(ids), 0
+        while live:
+            entries, row = [], 0
+            for r in live:
+                lo, hi = (0, prompt[r]) if t == 0 else (prompt[r] + t - 1, prompt[r] + t)
+                want = [i for i in range(hi - lo) if (lo + i) % 3 != 1]
+                entries.append({"id": r, "tokens": reqs[r][lo:hi], "want": want})
+                for i in want:
+                    where[r].append((n, row, lo + i))
+                    row += 1
+            ending = [r for r in live if prompt[r] + t >= len(reqs[r])]
+            steps.append({"step": n, "entries": entries, "end": ending})
+            live = [r for r in live if r not in ending]
+            n += 1
+            t += 1
+    lines = "\n".join(json.dumps(s) for s in steps) + "\n"
+    for dtype in ("float32", "bfloat16"):
+        out = str(tmp_path / dtype)
+        proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                               "--out", out, "--max-tokens", str(200 + 70)],
+                              input=lines, capture_output=True, text=True, timeout=110)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+        for r, toks in reqs.items():
+            want = P.forward(w, cfg, toks)
+            rows, places = [], []
+            for step, row, pos in where[r]:
+                data = np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, V)
+                rows.append(torch.from_numpy(data[row].copy()))
+                places.append(pos)
+            assert close(torch.stack(rows), want[places], dtype, TOL_F32_LONG), (dtype, r)
+        for s in steps:
+            if not any(e["want"] for e in s["entries"]):
+                assert not os.path.exists(os.path.join(out, f"{s['step']}.f32"))
