@@ -252,6 +252,300 @@ extern "C" int gfa_scored_attention(const void* q, const void* k_pages, const vo
 }
 
 // --------------------------------------------------------------------------------------
+// The same attention for bfloat16 on the matrix cores (head sizes in eights up to 576, value
+// sizes in sixteens up to 512).  A wave owns a tile of 16 rows, each a (token, head) pair of
+// one kv head, and walks the key blocks of 32 that its rows see.  Both products are formed
+// transposed, so that every operand is read in the order the cache has:
+//   S^T = K Q^T   A = 16 keys x 32 dims of a key page, B = Q^T from registers;
+//   O^T = V^T P^T A = 16 dims x 32 keys of a value page, B = the eight weights a lane holds.
+// v_mfma_f32_16x16x32_bf16: lane l supplies row (A) / column (B) l % 16, k = 8 (l / 16) .. +7,
+// and receives rows 4 (l / 16) .. +3 of column l % 16; with the key order of common.h those
+// rows of the two 16-key tiles are the lane's keys 8 (l / 16) .. +7 of the block.  Scores, the
+// steps on them, the softmax and both products' sums are float; the weights are rounded to
+// bfloat16 as the second product's operand.
+//
+// Without a mix across heads the waves of a workgroup are tiles of their own (grid: tiles / 4,
+// kv heads, sequences).  With one, the waves of a workgroup are the kv heads of one group of
+// tokens (a kv head with more than 16 heads takes several waves): every wave puts its tile of
+// scores into shared memory, and every lane adds up, for its row's head and its eight keys,
+// the scores of all heads of the same token.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 sa_bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float sa_floatx4_t;
+union SAFrag {
+    uint4 u;
+    bf16_t e[8];
+    sa_bf16x8_t v;
+};
+
+#define SA_SROW 36            // floats per row of a wave's score tile in shared memory (32 + 4)
+
+__device__ __forceinline__ float sa_max_lane_groups(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16, GFA_WAVE));
+    return fmaxf(v, __shfl_xor(v, 32, GFA_WAVE));
+}
+__device__ __forceinline__ float sa_sum_lane_groups(float v) {
+    v += __shfl_xor(v, 16, GFA_WAVE);
+    return v + __shfl_xor(v, 32, GFA_WAVE);
+}
+
+template <int DK, int DVT, int MAXT>
+__global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
+        const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+        const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
+        const int* __restrict__ start_pos, const int* __restrict__ table,
+        const float* __restrict__ temperature, const float* __restrict__ bias,
+        const int* __restrict__ lookup, const float* __restrict__ talk, bf16_t* __restrict__ out,
+        SAShape s) {
+    extern __shared__ __attribute__((aligned(16))) float sam_lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), nw = blockDim.x >> 6;
+    const int li = lane & 15, lg = lane >> 4;
+    const int seq = blockIdx.z;
+    const int gs = s.H / s.G;
+    const int q0 = q_start[seq], q_len = q_start[seq + 1] - q0;
+    const int spos = start_pos[seq];
+    const int* pages = table + (size_t)seq * s.table_stride;
+    const bool mix = talk != nullptr;
+
+    // which (token, head) this lane's row is, and which tokens the wave's rows span
+    int g, tok, head, tok_lo, tok_hi;
+    bool row_ok;
+    if (!mix) {
+        g = blockIdx.y;
+        const int rows_total = q_len * gs, row0 = (blockIdx.x * nw + wave) * 16;
+        if (row0 >= rows_total) return;                // no barrier follows without a mix
+        row_ok = row0 + li < rows_total;
+        const int row = row_ok ? row0 + li : rows_total - 1;
+        tok = row / gs;
+        head = g * gs + row % gs;
+        tok_lo = row0 / gs;
+        tok_hi = (row0 + 15 < rows_total ? row0 + 15 : rows_total - 1) / gs;
+    } else {
+        const int tpg = gs > 16 ? (gs + 15) / 16 : 1, tp = gs > 16 ? 1 : 16 / gs;
+        g = wave / tpg;
+        tok_lo = blockIdx.x * tp;
+        if (tok_lo >= q_len) return;                   // the whole workgroup
+        tok_hi = tok_lo + tp - 1 < q_len ? tok_lo + tp - 1 : q_len - 1;
+        int hg;
+        if (gs > 16) {
+            tok = tok_lo;
+            hg = (wave % tpg) * 16 + li;
+            row_ok = hg < gs;
+        } else {
+            tok = tok_lo + li / gs;
+            hg = li % gs;
+            row_ok = li < tp * gs && tok <= tok_hi;
+        }
+        if (!row_ok) {
+            tok = tok_lo;
+            hg = 0;
+        }
+        head = g * gs + hg;
+    }
+    const int pos = spos + tok;
+    const int lo = (s.window > 0 && pos - s.window + 1 > 0) ? pos - s.window + 1 : 0;
+    const int pos_max = spos + tok_hi;
+    const int lo_min = (s.window > 0 && spos + tok_lo - s.window + 1 > 0) ? spos + tok_lo - s.window + 1 : 0;
+    const int last_key = spos + q_len - 1;             // the newest key the cache holds of this sequence
+
+    float* talk_lds = sam_lds;                         // [H][H], with a mix
+    float* tiles = sam_lds + (mix ? s.H * s.H : 0);    // [waves][16][SA_SROW]
+    if (mix) {
+        for (int e = threadIdx.x; e < s.H * s.H; e += blockDim.x) talk_lds[e] = talk[e];
+        __syncthreads();
+    }
+
+    SAFrag qf[DK];
+    const bf16_t* qrow = q + (size_t)(q0 + tok) * s.q_tok + (size_t)head * s.q_head;
+#pragma unroll
+    for (int kk = 0; kk < DK; ++kk) {
+        const int d = kk * 32 + lg * 8;
+        qf[kk].u = d < s.hd ? *(const uint4*)(qrow + d) : make_uint4(0, 0, 0, 0);
+    }
+    const float row_scale = s.scale * (temperature ? temperature[head] : 1.f);
+    const int vtiles = s.vd / 16;
+    sa_floatx4_t o[DVT];
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt) o[dt] = sa_floatx4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    for (int bi = lo_min / 32; bi <= pos_max / 32; ++bi) {
+        const int page = pages[bi >> 1];
+        const bf16_t* kb = k_pages + cache_region(page, g, s.G, s.hd) + (size_t)(bi & 1) * 32 * s.hd;
+        const bf16_t* vb = v_pages + cache_region(page, g, s.G, s.vd) + (size_t)(bi & 1) * 512;
+        sa_floatx4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < DK; ++kk) {
+            const int chunk = kk * 4 + lg;
+            const int c = chunk * 8 < s.hd ? chunk : 0;          // q is zero there
+            const bf16_t* src = kb + c * 256 + li * 8;
+            SAFrag k0, k1;
+            k0.u = *(const uint4*)src;
+            k1.u = *(const uint4*)(src + 128);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0.v, qf[kk].v, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1.v, qf[kk].v, s1, 0, 0, 0);
+        }
+        float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+        const int key0 = bi * 32 + lg * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int j = key0 + e;
+            float v = sv[e] * row_scale;
+            if (s.softcap > 0.f) v = s.softcap * tanhf(v / s.softcap);
+            if (bias && j <= pos) {
+                const int dist = pos - j;
+                const int row = dist < s.n_lookup ? lookup[dist] : s.bias_rows - 1;
+                v += bias[(size_t)row * s.H + head];
+            }
+            // what lies beyond the newest key may be anything: it must not reach the mix
+            sv[e] = j <= last_key ? v : 0.f;
+        }
+        if (mix) {
+            float* mine = tiles + ((size_t)wave * 16 + li) * SA_SROW + lg * 8;
+            *(float4*)mine = make_float4(sv[0], sv[1], sv[2], sv[3]);
+            *(float4*)(mine + 4) = make_float4(sv[4], sv[5], sv[6], sv[7]);
+            __syncthreads();
+            float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            const float* trow = talk_lds + head * s.H;
+            // first row of this lane's token in a tile
+            const int tok_row = (gs > 16 || !row_ok) ? 0 : (li / gs) * gs;
+            const int tpg = gs > 16 ? (gs + 15) / 16 : 1;
+            for (int h2 = 0; h2 < s.H; ++h2) {
+                const int g2 = h2 / gs, r2 = h2 - g2 * gs;
+                const int w2 = g2 * tpg + (r2 >> 4);
+                const int row2 = gs > 16 ? (r2 & 15) : tok_row + r2;
+                const float* src = tiles + ((size_t)w2 * 16 + row2) * SA_SROW + lg * 8;
+                const float4 a = *(const float4*)src, b = *(const float4*)(src + 4);
+                const float t = trow[h2];
+                z[0] = fmaf(t, a.x, z[0]); z[1] = fmaf(t, a.y, z[1]);
+                z[2] = fmaf(t, a.z, z[2]); z[3] = fmaf(t, a.w, z[3]);
+                z[4] = fmaf(t, b.x, z[4]); z[5] = fmaf(t, b.y, z[5]);
+                z[6] = fmaf(t, b.z, z[6]); z[7] = fmaf(t, b.w, z[7]);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sv[e] = z[e];
+            __syncthreads();                           // the tiles are free for the next block
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int j = key0 + e;
+            sv[e] = (j <= pos && j >= lo) ? sv[e] * 1.4426950408889634f : -INFINITY;
+            mx = fmaxf(mx, sv[e]);
+        }
+        mx = sa_max_lane_groups(mx);
+        const float m_new = fmaxf(m, mx);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = exp2f(m - m_use);
+        SAFrag pf;
+        float ps = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float p = exp2f(sv[e] - m_use);
+            ps += p;
+            pf.e[e] = float_to_bf16(p);
+        }
+        l = l * alpha + ps;
+        m = m_new;
+        // values beyond the newest key: zero bits (their weight is zero, but the pool is not cleared)
+        auto two = [&](int e) {
+            return (key0 + e <= last_key ? 0xffffu : 0u) | (key0 + e + 1 <= last_key ? 0xffff0000u : 0u);
+        };
+        const uint4 keep = make_uint4(two(0), two(2), two(4), two(6));
+#pragma unroll
+        for (int dt = 0; dt < DVT; ++dt) {
+            const int dtc = dt < vtiles ? dt : vtiles - 1;
+            SAFrag vf;
+            vf.u = *(const uint4*)(vb + (size_t)dtc * 1024 + lg * 128 + li * 8);
+            vf.u.x &= keep.x;
+            vf.u.y &= keep.y;
+            vf.u.z &= keep.z;
+            vf.u.w &= keep.w;
+            o[dt] *= alpha;
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
+        }
+    }
+    l = sa_sum_lane_groups(l);
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    if (!row_ok) return;
+    bf16_t* orow = out + (size_t)(q0 + tok) * s.o_tok + (size_t)head * s.o_head;
+#pragma unroll
+    for (int dt = 0; dt < DVT; ++dt) {
+        if (dt < vtiles) {
+            const uint32_t a = (uint32_t)float_to_bf16(o[dt][0] * inv) | ((uint32_t)float_to_bf16(o[dt][1] * inv) << 16);
+            const uint32_t b = (uint32_t)float_to_bf16(o[dt][2] * inv) | ((uint32_t)float_to_bf16(o[dt][3] * inv) << 16);
+            uint32_t* dst = (uint32_t*)(orow + dt * 16 + lg * 4);
+            dst[0] = a;
+            dst[1] = b;
+        }
+    }
+}
+
+template <int DK, int DVT, int MAXT>
+static int sam_launch(const void* q, const void* k_pages, const void* v_pages, const int* q_start,
+                      const int* start_pos, const int* table, const float* temperature,
+                      const float* bias, const int* lookup, const float* talk, void* out,
+                      int n_seqs, int max_q_len, const SAShape& s, hipStream_t stream) {
+    const int gs = s.H / s.G;
+    dim3 grid, block;
+    size_t shmem = 0;
+    if (talk) {
+        const int tpg = gs > 16 ? (gs + 15) / 16 : 1, tp = gs > 16 ? 1 : 16 / gs;
+        const int waves = s.G * tpg;
+        if (waves * 64 > MAXT) return (int)hipErrorInvalidValue;
+        grid = dim3((max_q_len + tp - 1) / tp, 1, n_seqs);
+        block = dim3(waves * 64);
+        shmem = sizeof(float) * ((size_t)s.H * s.H + (size_t)waves * 16 * SA_SROW);
+        if (shmem > 64 * 1024) return (int)hipErrorInvalidValue;
+    } else {
+        const int tiles = (max_q_len * gs + 15) / 16;
+        grid = dim3((tiles + 3) / 4, s.G, n_seqs);
+        block = dim3(256);
+    }
+    scored_attention_mfma_kernel<DK, DVT, MAXT><<<grid, block, shmem, stream>>>(
+        (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table,
+        temperature, bias, lookup, talk, (bf16_t*)out, s);
+    return GFA_LAUNCH_RESULT();
+}
+
+// 1 if the matrix-core kernel takes these sizes (bfloat16 only)
+extern "C" int gfa_scored_attention_mfma_takes(int H, int G, int hd, int vd, int mixed) {
+    if (G <= 0 || H % G || hd % 8 || vd % 16 || hd > 576 || vd > 512 || hd < 8) return 0;
+    if (mixed) {
+        const int gs = H / G;
+        const int waves = G * (gs > 16 ? (gs + 15) / 16 : 1);
+        if (H > 64 || (gs <= 16 && 16 / gs < 1)) return 0;
+        const bool small = hd <= 128 && vd <= 128;
+        if (waves > (small ? 16 : 4)) return 0;
+        if (sizeof(float) * ((size_t)H * H + (size_t)waves * 16 * SA_SROW) > 64 * 1024) return 0;
+    }
+    return 1;
+}
+
+extern "C" int gfa_scored_attention_mfma(const void* q, const void* k_pages, const void* v_pages,
+                                         const int* q_start, const int* start_pos, const int* table,
+                                         int table_stride, const float* temperature,
+                                         const float* bias, const int* lookup, const float* talk,
+                                         void* out, int n_seqs, int max_q_len, int H, int G, int hd,
+                                         int vd, long long q_tok, long long q_head, long long o_tok,
+                                         long long o_head, float scale, float softcap, int bias_rows,
+                                         int n_lookup, int window, hipStream_t stream) {
+    if (n_seqs <= 0 || max_q_len <= 0) return 0;
+    if (!gfa_scored_attention_mfma_takes(H, G, hd, vd, talk != nullptr) || n_seqs > 65535)
+        return (int)hipErrorInvalidValue;
+    // 16-byte loads of q, 4-byte stores of the result
+    if (q_tok % 8 || q_head % 8 || o_tok % 2 || o_head % 2) return (int)hipErrorInvalidValue;
+    SAShape s{H, G, hd, vd, q_tok, q_head, o_tok, o_head, table_stride, window, scale, softcap,
+              bias_rows, n_lookup};
+#define SAM_GO(DK, DVT, MAXT) return sam_launch<DK, DVT, MAXT>(q, k_pages, v_pages, q_start, start_pos, \
+        table, temperature, bias, lookup, talk, out, n_seqs, max_q_len, s, stream)
+    if (hd <= 128 && vd <= 128) SAM_GO(4, 8, 1024);
+    if (hd <= 256 && vd <= 256) SAM_GO(8, 16, 256);
+    SAM_GO(18, 32, 256);
+#undef SAM_GO
+}
+
+// --------------------------------------------------------------------------------------
 // q, keys and values of attention with unit-norm heads from the projection's float sums:
 // a row of proj is [H heads of q | G heads of k | G heads of v] (d, d, dv wide); the bias
 // (same layout, optional) is added first; every head of q and k is divided by its root mean

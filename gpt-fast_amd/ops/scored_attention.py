@@ -52,13 +52,15 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tok
               scale: float, *, window: int = 0, temperature: Optional[torch.Tensor] = None,
               softcap: float = 0.0, bias: Optional[torch.Tensor] = None,
               lookup: Optional[torch.Tensor] = None, talk: Optional[torch.Tensor] = None,
-              head_major: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+              head_major: bool = False, out: Optional[torch.Tensor] = None, step=None) -> torch.Tensor:
     """Each token's heads attend to the keys of its sequence's pages.  q is [N, H, hd], or
     [H, N, hd] if ``head_major`` (the result then lies the same way); k_pages
     [pages, G, 64, hd], v_pages [pages, G, vd, 64]; temperature float32 [H]; bias float32
     [rows, H] with lookup int32 [distances] (see :func:`distance_rows`); talk float32 [H, H].
     Returns [N, H, vd] (or [H, N, vd]) in q's type.  ``out`` may be a view with unit stride
-    in its last dimension."""
+    in its last dimension.  ``step`` = (q_start int32 [B + 1], start_pos int32 [B], B, longest
+    run of new tokens) describes the same tokens sequence by sequence; with it, bfloat16 rows
+    of sizes the matrix-core kernel takes go there."""
     require_device(q, k_pages, v_pages, tok_seq, tok_pos, table, temperature, bias, lookup, talk, out)
     require_contiguous(tok_seq=tok_seq, tok_pos=tok_pos, table=table, temperature=temperature,
                        bias=bias, lookup=lookup, talk=talk)
@@ -95,7 +97,26 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tok
     elif tuple(out.shape) != shape or out.dtype != q.dtype or out.stride(2) != 1:
         raise KernelError("scored attention: out has the wrong shape, type or strides")
     tok, head = (1, 0) if head_major else (0, 1)
-    check(library("scored_attention").gfa_scored_attention(
+    lib = library("scored_attention")
+    if (step is not None and q.dtype == torch.bfloat16 and q.data_ptr() % 16 == 0
+            and out.data_ptr() % 4 == 0 and q.stride(tok) % 8 == 0 and q.stride(head) % 8 == 0
+            and out.stride(tok) % 2 == 0 and out.stride(head) % 2 == 0
+            and lib.gfa_scored_attention_mfma_takes(_i(H), _i(G), _i(hd), _i(vd), _i(int(talk is not None)))):
+        q_start, start_pos, n_seqs, max_q_len = step
+        require_device(q_start, start_pos)
+        require_contiguous(q_start=q_start, start_pos=start_pos)
+        if q_start.dtype != torch.int32 or start_pos.dtype != torch.int32 or \
+                q_start.numel() < n_seqs + 1 or start_pos.numel() < n_seqs:
+            raise KernelError("scored attention: q_start / start_pos must be int32 and cover the batch")
+        check(lib.gfa_scored_attention_mfma(
+            ptr(q), ptr(k_pages), ptr(v_pages), ptr(q_start), ptr(start_pos), ptr(table),
+            _i(table.shape[1]), ptr(temperature), ptr(bias), ptr(lookup if bias is not None else None),
+            ptr(talk), ptr(out), _i(n_seqs), _i(max_q_len), _i(H), _i(G), _i(hd), _i(vd),
+            _ll(q.stride(tok)), _ll(q.stride(head)), _ll(out.stride(tok)), _ll(out.stride(head)),
+            _f(scale), _f(softcap or 0.0), _i(rows), _i(0 if lookup is None else lookup.numel()),
+            _i(window or 0), stream_handle()), "scored_attention_mfma")
+        return out
+    check(lib.gfa_scored_attention(
         ptr(q), ptr(k_pages), ptr(v_pages), ptr(tok_seq), ptr(tok_pos), ptr(table),
         _i(table.shape[1]), ptr(temperature), ptr(bias), ptr(lookup if bias is not None else None),
         ptr(talk), ptr(out), _i(n), _i(H), _i(G), _i(hd), _i(vd), _ll(q.stride(tok)),

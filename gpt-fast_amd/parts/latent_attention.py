@@ -117,7 +117,8 @@ class LatentAttention(Part):
 
         def finish(rows, then_norm, takes_halves):
             latent = SA.attention(full, entry.k_pages, entry.v_pages, batch.tok_seq, batch.tok_pos,
-                                  table, s.scale, window=self.window, head_major=True)
+                                  table, s.scale, window=self.window, head_major=True,
+                                  step=(batch.q_start, batch.start_pos, batch.n_seqs, batch.max_q_len))
             y = torch.empty((n, s.n_heads, s.value_dim), dtype=self.rt.dtype, device=x.device)
             self._per_head(latent, self.w_uv, y.permute(1, 0, 2))
             return L.linear_into(y.view(n, s.n_heads * s.value_dim), self.wo, rows, then_norm,

@@ -87,7 +87,8 @@ class MixedHeadsAttention(Part):
         def finish(rows, then_norm, takes_halves):
             y = SA.attention(q, entry.k_pages, entry.v_pages, batch.tok_seq, batch.tok_pos, table,
                              s.scale, temperature=self.temperature, softcap=s.softcap or 0.0,
-                             bias=self.bias, lookup=self.lookup, talk=self.talk)
+                             bias=self.bias, lookup=self.lookup, talk=self.talk,
+                             step=(batch.q_start, batch.start_pos, batch.n_seqs, batch.max_q_len))
             out = L.linear_into(y.view(q.shape[0], s.n_heads * s.value_dim), self.wo, rows,
                                 then_norm, takes_halves)
             if self.bo is not None:
