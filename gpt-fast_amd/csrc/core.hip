@@ -764,17 +764,92 @@ __global__ __launch_bounds__(256) void normed_add_kernel(
     for (int d = threadIdx.x; d < dim; d += 256) store_from_float(o + d, rr[d] * rn * next_w[d]);
 }
 
+// The same for rows of up to 1024 * VPT * 4 elements (a multiple of 4): y and the stream are
+// read once with 16-byte loads and kept in registers between the sums and the stores.
+template <typename T, int VPT, int THREADS>
+__global__ __launch_bounds__(THREADS) void normed_add_vec_kernel(
+        float* __restrict__ res, const float* __restrict__ y, const float* __restrict__ wy,
+        float eps_y, const float* __restrict__ next_w, float eps_n, T* __restrict__ out, int dim) {
+    __shared__ float scratch[16];
+    const size_t row = (size_t)blockIdx.x * dim;
+    const float4* y4 = (const float4*)(y + row);
+    float4* r4 = (float4*)(res + row);
+    const float4* wy4 = (const float4*)wy;
+    const int n4 = dim >> 2;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 yv[VPT], rv[VPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        yv[j] = idx < n4 ? y4[idx] : zero;
+        rv[j] = idx < n4 ? r4[idx] : zero;
+        ss = fmaf(yv[j].x, yv[j].x, ss);
+        ss = fmaf(yv[j].y, yv[j].y, ss);
+        ss = fmaf(yv[j].z, yv[j].z, ss);
+        ss = fmaf(yv[j].w, yv[j].w, ss);
+    }
+    ss = block_sum(ss, scratch);
+    const float ry = rsqrtf(ss / (float)dim + eps_y);
+    float sn = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        if (idx < n4) {
+            const float4 g = wy4[idx];
+            rv[j].x += yv[j].x * ry * g.x;
+            rv[j].y += yv[j].y * ry * g.y;
+            rv[j].z += yv[j].z * ry * g.z;
+            rv[j].w += yv[j].w * ry * g.w;
+            r4[idx] = rv[j];
+            sn = fmaf(rv[j].x, rv[j].x, sn);
+            sn = fmaf(rv[j].y, rv[j].y, sn);
+            sn = fmaf(rv[j].z, rv[j].z, sn);
+            sn = fmaf(rv[j].w, rv[j].w, sn);
+        }
+    }
+    if (next_w == nullptr) return;
+    sn = block_sum(sn, scratch);
+    const float rn = rsqrtf(sn / (float)dim + eps_n);
+    const float4* nw4 = (const float4*)next_w;
+    T* o = out + row;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+        const int idx = threadIdx.x + j * THREADS;
+        if (idx < n4) {
+            const float4 g = nw4[idx];
+            store_from_float(o + 4 * idx + 0, rv[j].x * rn * g.x);
+            store_from_float(o + 4 * idx + 1, rv[j].y * rn * g.y);
+            store_from_float(o + 4 * idx + 2, rv[j].z * rn * g.z);
+            store_from_float(o + 4 * idx + 3, rv[j].w * rn * g.w);
+        }
+    }
+}
+
+template <typename T>
+static int launch_normed_add(float* res, const float* y, const float* wy, float eps_y,
+                             const float* next_w, float eps_n, T* out, int n_rows, int dim,
+                             hipStream_t stream) {
+    if (dim % 4 == 0 && dim <= 8192) {
+        if (dim <= 1024)
+            normed_add_vec_kernel<T, 1, 256><<<n_rows, 256, 0, stream>>>(res, y, wy, eps_y, next_w, eps_n, out, dim);
+        else if (dim <= 4096)
+            normed_add_vec_kernel<T, 1, 1024><<<n_rows, 1024, 0, stream>>>(res, y, wy, eps_y, next_w, eps_n, out, dim);
+        else
+            normed_add_vec_kernel<T, 2, 1024><<<n_rows, 1024, 0, stream>>>(res, y, wy, eps_y, next_w, eps_n, out, dim);
+    } else {
+        normed_add_kernel<T><<<n_rows, 256, 0, stream>>>(res, y, wy, eps_y, next_w, eps_n, out, dim);
+    }
+    return GFA_LAUNCH_RESULT();
+}
+
 extern "C" int gfa_normed_add(float* res, const float* y, const float* wy, float eps_y,
                               const float* next_w, float eps_n, void* out, int out_bf16,
                               int n_rows, int dim, hipStream_t stream) {
     if (n_rows <= 0) return 0;
     if (out_bf16)
-        normed_add_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(res, y, wy, eps_y, next_w, eps_n,
-                                                             (bf16_t*)out, dim);
-    else
-        normed_add_kernel<float><<<n_rows, 256, 0, stream>>>(res, y, wy, eps_y, next_w, eps_n,
-                                                            (float*)out, dim);
-    return GFA_LAUNCH_RESULT();
+        return launch_normed_add<bf16_t>(res, y, wy, eps_y, next_w, eps_n, (bf16_t*)out, n_rows, dim, stream);
+    return launch_normed_add<float>(res, y, wy, eps_y, next_w, eps_n, (float*)out, n_rows, dim, stream);
 }
 
 // --------------------------------------------------------------------------------------

@@ -288,7 +288,7 @@ __device__ __forceinline__ float sa_sum_lane_groups(float v) {
     return v + __shfl_xor(v, 32, GFA_WAVE);
 }
 
-template <int DK, int DVT, int MAXT>
+template <int DK, int DVT, int MAXT, bool SPLIT>
 __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
         const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
         const bf16_t* __restrict__ v_pages, const int* __restrict__ q_start,
@@ -312,8 +312,8 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
     bool row_ok;
     if (!mix) {
         g = blockIdx.y;
-        const int rows_total = q_len * gs, row0 = (blockIdx.x * nw + wave) * 16;
-        if (row0 >= rows_total) return;                // no barrier follows without a mix
+        const int rows_total = q_len * gs, row0 = (SPLIT ? blockIdx.x : blockIdx.x * nw + wave) * 16;
+        if (row0 >= rows_total) return;                // SPLIT: the whole workgroup; else no barrier follows
         row_ok = row0 + li < rows_total;
         const int row = row_ok ? row0 + li : rows_total - 1;
         tok = row / gs;
@@ -369,7 +369,8 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
     for (int dt = 0; dt < DVT; ++dt) o[dt] = sa_floatx4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    for (int bi = lo_min / 32; bi <= pos_max / 32; ++bi) {
+    // SPLIT: the waves of a workgroup share one tile of rows and take its key blocks in turn
+    for (int bi = lo_min / 32 + (SPLIT ? wave : 0); bi <= pos_max / 32; bi += SPLIT ? nw : 1) {
         const int page = pages[bi >> 1];
         const bf16_t* kb = k_pages + cache_region(page, g, s.G, s.hd) + (size_t)(bi & 1) * 32 * s.hd;
         const bf16_t* vb = v_pages + cache_region(page, g, s.G, s.vd) + (size_t)(bi & 1) * 512;
@@ -466,6 +467,40 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
         }
     }
     l = sa_sum_lane_groups(l);
+    if (SPLIT) {
+        // per wave: m and l of its 16 rows, then O^T [dim][row]; the first wave adds them up in
+        // wave order (the maxima are in units of log 2)
+        const int per_wave = 32 + s.vd * 16;
+        float* mine = sam_lds + (size_t)wave * per_wave;
+        if (lg == 0) {
+            mine[li] = m;
+            mine[16 + li] = l;
+        }
+#pragma unroll
+        for (int dt = 0; dt < DVT; ++dt)
+            if (dt < vtiles)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) mine[32 + (dt * 16 + lg * 4 + j) * 16 + li] = o[dt][j];
+        __syncthreads();
+        if (wave != 0) return;
+        float M = -INFINITY;
+        for (int w = 0; w < nw; ++w) M = fmaxf(M, sam_lds[(size_t)w * per_wave + li]);
+        l = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DVT; ++dt) o[dt] = sa_floatx4_t{0.f, 0.f, 0.f, 0.f};
+        for (int w = 0; w < nw; ++w) {
+            const float* theirs = sam_lds + (size_t)w * per_wave;
+            const float mw = theirs[li];
+            const float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
+            l = fmaf(theirs[16 + li], f, l);
+#pragma unroll
+            for (int dt = 0; dt < DVT; ++dt)
+                if (dt < vtiles)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        o[dt][j] = fmaf(theirs[32 + (dt * 16 + lg * 4 + j) * 16 + li], f, o[dt][j]);
+        }
+    }
     const float inv = l > 0.f ? 1.f / l : 0.f;
     if (!row_ok) return;
     bf16_t* orow = out + (size_t)(q0 + tok) * s.o_tok + (size_t)head * s.o_head;
@@ -481,7 +516,7 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
     }
 }
 
-template <int DK, int DVT, int MAXT>
+template <int DK, int DVT, int MAXT, bool SPLIT>
 static int sam_launch(const void* q, const void* k_pages, const void* v_pages, const int* q_start,
                       const int* start_pos, const int* table, const float* temperature,
                       const float* bias, const int* lookup, const float* talk, void* out,
@@ -497,12 +532,27 @@ static int sam_launch(const void* q, const void* k_pages, const void* v_pages, c
         block = dim3(waves * 64);
         shmem = sizeof(float) * ((size_t)s.H * s.H + (size_t)waves * 16 * SA_SROW);
         if (shmem > 64 * 1024) return (int)hipErrorInvalidValue;
+    } else if (SPLIT) {
+        // as many waves as their partial results fit the shared memory a workgroup may have
+        const int waves = s.vd > 256 ? 4 : 8;
+        if (waves * 64 > MAXT) return (int)hipErrorInvalidValue;
+        grid = dim3((max_q_len * gs + 15) / 16, s.G, n_seqs);
+        block = dim3(waves * 64);
+        shmem = sizeof(float) * (size_t)waves * (32 + (size_t)s.vd * 16);
+        static bool allowed = false;
+        if (!allowed) {
+            const hipError_t e = hipFuncSetAttribute(
+                (const void*)scored_attention_mfma_kernel<DK, DVT, MAXT, SPLIT>,
+                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return (int)e;
+            allowed = true;
+        }
     } else {
         const int tiles = (max_q_len * gs + 15) / 16;
         grid = dim3((tiles + 3) / 4, s.G, n_seqs);
         block = dim3(256);
     }
-    scored_attention_mfma_kernel<DK, DVT, MAXT><<<grid, block, shmem, stream>>>(
+    scored_attention_mfma_kernel<DK, DVT, MAXT, SPLIT><<<grid, block, shmem, stream>>>(
         (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, q_start, start_pos, table,
         temperature, bias, lookup, talk, (bf16_t*)out, s);
     return GFA_LAUNCH_RESULT();
@@ -537,11 +587,17 @@ extern "C" int gfa_scored_attention_mfma(const void* q, const void* k_pages, con
     if (q_tok % 8 || q_head % 8 || o_tok % 2 || o_head % 2) return (int)hipErrorInvalidValue;
     SAShape s{H, G, hd, vd, q_tok, q_head, o_tok, o_head, table_stride, window, scale, softcap,
               bias_rows, n_lookup};
-#define SAM_GO(DK, DVT, MAXT) return sam_launch<DK, DVT, MAXT>(q, k_pages, v_pages, q_start, start_pos, \
-        table, temperature, bias, lookup, talk, out, n_seqs, max_q_len, s, stream)
-    if (hd <= 128 && vd <= 128) SAM_GO(4, 8, 1024);
-    if (hd <= 256 && vd <= 256) SAM_GO(8, 16, 256);
-    SAM_GO(18, 32, 256);
+#define SAM_GO(DK, DVT, MAXT, SPLIT) return sam_launch<DK, DVT, MAXT, SPLIT>(q, k_pages, v_pages, q_start, \
+        start_pos, table, temperature, bias, lookup, talk, out, n_seqs, max_q_len, s, stream)
+    // one token per sequence and no mix: the waves of a workgroup share a tile's key blocks
+    if (max_q_len == 1 && talk == nullptr) {
+        if (hd <= 128 && vd <= 128) SAM_GO(4, 8, 512, true);
+        if (hd <= 256 && vd <= 256) SAM_GO(8, 16, 512, true);
+        SAM_GO(18, 32, 512, true);
+    }
+    if (hd <= 128 && vd <= 128) SAM_GO(4, 8, 1024, false);
+    if (hd <= 256 && vd <= 256) SAM_GO(8, 16, 256, false);
+    SAM_GO(18, 32, 256, false);
 #undef SAM_GO
 }
 

@@ -87,7 +87,7 @@ def test_activation_kernel():
 def test_a_result_joins_the_stream_through_its_norm():
     from gpt_fast_amd.ops import kernels as K
     torch.manual_seed(1)
-    for dim in (50, 96, 1030):
+    for dim in (50, 96, 1030, 2048, 4096, 6144):
         res = torch.randn(9, dim, device=DEV) * 2
         y = torch.randn(9, dim, device=DEV) * 5
         w1, w2 = torch.randn(dim, device=DEV), torch.randn(dim, device=DEV)
@@ -296,6 +296,16 @@ def test_scored_attention_alone(dtype, tol, H, G, d, dv, window, mixed, head_maj
     err = _scored_attention_alone(dtype, H, G, d, dv, window, lens=[130, 40, 1, 1, 3], starts=[0, 70, 200, 0, 63],
                                   mixed=mixed, head_major=head_major, by_sequence=by_sequence)
     assert err < tol
+
+
+@pytest.mark.parametrize("H,G,d,dv,window", [(3, 1, 40, 32, 24), (32, 1, 576, 512, 300), (4, 1, 160, 144, 70),
+                                             (40, 1, 72, 64, None), (4, 2, 64, 64, 33), (8, 8, 128, 128, None)])
+def test_single_token_steps_share_their_key_blocks_among_waves(H, G, d, dv, window):
+    """One token per sequence, no mix: sequences of one key, of less than a block, of several
+    pages; fewer blocks than waves and more."""
+    err = _scored_attention_alone(torch.bfloat16, H, G, d, dv, window, lens=[1, 1, 1, 1, 1, 1],
+                                  starts=[0, 5, 31, 32, 200, 700], mixed=False, head_major=G == 1, by_sequence=True)
+    assert err < 2e-2
 
 
 @pytest.mark.parametrize("window,key", [(24, 176), (24, 175), (64, 136), (64, 135), (100, 100), (100, 99)])
