@@ -12,7 +12,8 @@ the live sequences) per second with the HBM peak; ``points`` holds decode at bat
 
 Other workloads of the same program: ``--preset`` (another shape, also of another
 architecture: ``pigodra-4096`` is a Pigodra stack with the width, inner size and head sizes of
-``llama-3.1-8b``; with ``--layers N`` both run their first N layers), ``--context`` (cache
+``llama-3.1-8b``, ``nizedra-4096`` a Nizedra stack of that width and as many weights per layer;
+with ``--layers N`` all run their first N layers), ``--context`` (cache
 positions per sequence), ``--prompt-lens LO:HI`` (prompts of unequal, seeded random lengths;
 adds the ragged prefill's tokens per second), ``--prefill-only`` (just the timed prompt, for
 profiling), ``--parts`` (no model: a layer's products at ``--batch`` rows and the prompt

@@ -355,17 +355,17 @@ extern "C" int gfa_decayed_memory_chunks(const float* proj, const float* decay, 
 //     y[t, :] = o[t, :] * rsqrt(mean(o[t, :]^2) + eps) * weight[:] * sigmoid(gate[t, :])
 // The gate's pre-activations lie in proj at column g_off.  One workgroup per token.
 template <typename T>
-__global__ __launch_bounds__(256) void row_norm_gate_kernel(
+__global__ __launch_bounds__(1024) void row_norm_gate_kernel(
         const float* __restrict__ o, const float* __restrict__ weight, const float* __restrict__ proj,
         int row_width, int g_off, T* __restrict__ y, int width, float eps) {
     __shared__ float scratch[16];
     const size_t t = blockIdx.x;
     const float* src = o + t * width;
     float ss = 0.f;
-    for (int d = threadIdx.x; d < width; d += 256) ss = fmaf(src[d], src[d], ss);
+    for (int d = threadIdx.x; d < width; d += blockDim.x) ss = fmaf(src[d], src[d], ss);
     const float r = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
     const float* gate = proj + t * row_width + g_off;
-    for (int d = threadIdx.x; d < width; d += 256)
+    for (int d = threadIdx.x; d < width; d += blockDim.x)
         store_from_float(y + t * width + d, src[d] * r * weight[d] / (1.f + expf(-gate[d])));
 }
 
@@ -373,11 +373,12 @@ extern "C" int gfa_row_norm_gate(const float* o, const float* weight, const floa
                                  int row_width, int g_off, void* y, int y_bf16, int n_tokens,
                                  int width, float eps, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    const int threads = width > 1024 ? 1024 : 256;       // an element or a few per thread
     if (y_bf16)
-        row_norm_gate_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(o, weight, proj, row_width, g_off,
-                                                                  (bf16_t*)y, width, eps);
+        row_norm_gate_kernel<bf16_t><<<n_tokens, threads, 0, stream>>>(o, weight, proj, row_width, g_off,
+                                                                      (bf16_t*)y, width, eps);
     else
-        row_norm_gate_kernel<float><<<n_tokens, 256, 0, stream>>>(o, weight, proj, row_width, g_off,
-                                                                 (float*)y, width, eps);
+        row_norm_gate_kernel<float><<<n_tokens, threads, 0, stream>>>(o, weight, proj, row_width, g_off,
+                                                                     (float*)y, width, eps);
     return GFA_LAUNCH_RESULT();
 }

@@ -46,7 +46,7 @@ def _int_or_str(x):
 
 def build_parser() -> argparse.ArgumentParser:
     p = argparse.ArgumentParser(prog="gpt_fast_amd", description="Generate with a model of a "
-                                "registered architecture (Llama, Pigodra) on an MI355X.")
+                                "registered architecture (Llama, Pigodra, Nizedra) on an MI355X.")
     p.add_argument("--prompt", type=_int_or_str, default="Hello, my name is",
                    help="Input prompt. If it's an integer, will instead generate a synthetic prompt.")
     p.add_argument("--prompt_ids", type=str, default=None,

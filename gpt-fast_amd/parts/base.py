@@ -12,6 +12,9 @@ Interfaces (N = tokens of the step, D = model width):
                  ``forward(x [N, D], batch, entry, residual)`` adds its output into
                  ``residual`` (float32 [N, D], in place)
 * feed-forward:  ``forward(x [N, D], batch, residual)`` adds its output into ``residual``
+                 (a mixer or feed-forward may also offer ``forward_rows(x, batch[, entry]) ->
+                 float32 [N, D]``, its output alone, for blocks that treat it before it joins
+                 the stream)
 * position:      ``rotate_and_store(qkv, batch, entry, n_heads, n_kv_heads, head_dim) -> q``
 * block:         ``forward(residual, batch, entry)`` updates ``residual`` in place
 * stream step:   ``forward(residual float32 [N, D], embedded float32 [N, D], batch) ->`` the new

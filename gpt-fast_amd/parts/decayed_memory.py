@@ -61,14 +61,21 @@ class DecayedMemory(Part):
         cell = 2.0 * 2.0 * s.n_heads * s.key_dim * s.value_dim          # update and read of S
         return n * (2.0 * (self.in_rows + s.n_heads * s.value_dim) * s.dim + cell)
 
-    def forward(self, x, batch, entry, residual):
+    def _gated(self, x, batch, entry):
         s = self.spec
         proj = L.linear(x, self.w_in, out_dtype=torch.float32)
         o = M.cell(proj, self.rows, self.decay, entry.state, batch.q_start, batch.slots,
                    batch.n_seqs, batch.max_q_len, s.n_heads, s.key_dim, s.value_dim)
-        y = M.row_norm_gate(o, self.norm, proj, self.rows, s.eps, self.rt.dtype)
+        return M.row_norm_gate(o, self.norm, proj, self.rows, s.eps, self.rt.dtype)
+
+    def forward(self, x, batch, entry, residual):
+        y = self._gated(x, batch, entry)
         add_late(residual, lambda rows, then_norm, takes_halves: L.linear_into(
             y, self.wo, rows, then_norm, takes_halves))
+
+    def forward_rows(self, x, batch, entry):
+        """The mixer's output alone: the output projection's float32 sums."""
+        return L.linear(self._gated(x, batch, entry), self.wo, out_dtype=torch.float32)
 
 
 register_mixer("decayed_memory", DecayedMemory)

@@ -87,12 +87,17 @@ class DenseFeedForward(Part):
     def step_flops(self, q_lens, starts) -> float:
         return 2.0 * sum(q_lens) * 2 * self.spec.hidden * self.spec.dim
 
+    def _inner(self, x):
+        h = L.linear(x, self.w_up)
+        return K.activate(h, self.spec.activation, self.a, self.b, out=h)
+
     def forward(self, x, batch, residual):
-        def finish(rows, then_norm, takes_halves):
-            h = L.linear(x, self.w_up)
-            K.activate(h, self.spec.activation, self.a, self.b, out=h)
-            return L.linear_into(h, self.w_down, rows, then_norm, takes_halves)
-        add_late(residual, finish)
+        add_late(residual, lambda rows, then_norm, takes_halves: L.linear_into(
+            self._inner(x), self.w_down, rows, then_norm, takes_halves))
+
+    def forward_rows(self, x, batch):
+        """The feed-forward's output alone: the second product's float32 sums."""
+        return L.linear(self._inner(x), self.w_down, out_dtype=torch.float32)
 
 
 register_feed_forward("dense", DenseFeedForward)

@@ -96,7 +96,7 @@ class LatentAttention(Part):
             return K.gemm_f32_batched(a, w, out)
         return torch.bmm(a, w.transpose(1, 2), out=out)        # the vendor library, as for prompts
 
-    def forward(self, x, batch, entry, residual):
+    def _heads(self, x, batch, entry):
         s = self.spec
         n = x.shape[0]
         R = s.kv_rank
@@ -114,17 +114,21 @@ class LatentAttention(Part):
                                       s.head_dim, s.rot_dim, R, self.rt.dtype)
         # w_uk[h] is [d, R]: as the second operand it is taken transposed, [R, d]
         self._per_head(plain, self.w_uk.transpose(1, 2), full[:, :, :R])
+        latent = SA.attention(full, entry.k_pages, entry.v_pages, batch.tok_seq, batch.tok_pos,
+                              table, s.scale, window=self.window, head_major=True,
+                              step=(batch.q_start, batch.start_pos, batch.n_seqs, batch.max_q_len))
+        y = torch.empty((n, s.n_heads, s.value_dim), dtype=self.rt.dtype, device=x.device)
+        self._per_head(latent, self.w_uv, y.permute(1, 0, 2))
+        return y.view(n, s.n_heads * s.value_dim)
 
-        def finish(rows, then_norm, takes_halves):
-            latent = SA.attention(full, entry.k_pages, entry.v_pages, batch.tok_seq, batch.tok_pos,
-                                  table, s.scale, window=self.window, head_major=True,
-                                  step=(batch.q_start, batch.start_pos, batch.n_seqs, batch.max_q_len))
-            y = torch.empty((n, s.n_heads, s.value_dim), dtype=self.rt.dtype, device=x.device)
-            self._per_head(latent, self.w_uv, y.permute(1, 0, 2))
-            return L.linear_into(y.view(n, s.n_heads * s.value_dim), self.wo, rows, then_norm,
-                                 takes_halves)
+    def forward(self, x, batch, entry, residual):
+        y = self._heads(x, batch, entry)
+        add_late(residual, lambda rows, then_norm, takes_halves: L.linear_into(
+            y, self.wo, rows, then_norm, takes_halves))
 
-        add_late(residual, finish)
+    def forward_rows(self, x, batch, entry):
+        """The mixer's output alone: the output projection's float32 sums."""
+        return L.linear(self._heads(x, batch, entry), self.wo, out_dtype=torch.float32)
 
 
 register_mixer("latent_attention", LatentAttention)

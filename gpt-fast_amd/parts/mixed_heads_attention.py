@@ -74,7 +74,7 @@ class MixedHeadsAttention(Part):
             flops += 2.0 * per_key * keys
         return flops
 
-    def forward(self, x, batch, entry, residual):
+    def _heads(self, x, batch, entry):
         s = self.spec
         proj = L.linear(x, self.wqkv, out_dtype=torch.float32)
         write = entry is not None and entry.writes
@@ -83,21 +83,28 @@ class MixedHeadsAttention(Part):
                                 entry.k_pages if write else None, entry.v_pages if write else None,
                                 s.n_heads, s.n_kv_heads, s.head_dim, s.value_dim, s.qk_norm_eps,
                                 self.rt.dtype)
+        y = SA.attention(q, entry.k_pages, entry.v_pages, batch.tok_seq, batch.tok_pos, table,
+                         s.scale, temperature=self.temperature, softcap=s.softcap or 0.0,
+                         bias=self.bias, lookup=self.lookup, talk=self.talk,
+                         step=(batch.q_start, batch.start_pos, batch.n_seqs, batch.max_q_len))
+        return y.view(q.shape[0], s.n_heads * s.value_dim)
+
+    def forward(self, x, batch, entry, residual):
+        y = self._heads(x, batch, entry)
 
         def finish(rows, then_norm, takes_halves):
-            y = SA.attention(q, entry.k_pages, entry.v_pages, batch.tok_seq, batch.tok_pos, table,
-                             s.scale, temperature=self.temperature, softcap=s.softcap or 0.0,
-                             bias=self.bias, lookup=self.lookup, talk=self.talk,
-                             step=(batch.q_start, batch.start_pos, batch.n_seqs, batch.max_q_len))
-            out = L.linear_into(y.view(q.shape[0], s.n_heads * s.value_dim), self.wo, rows,
-                                then_norm, takes_halves)
+            # the bias joins after the product: no norm can ride on the product's kernel
+            L.linear_into(y, self.wo, rows, None if self.bo is not None else then_norm, takes_halves)
             if self.bo is not None:
-                if out is not None:
-                    raise RuntimeError("a norm was made before the output's bias was added")
                 K.add_bias(rows, self.bo)
-            return out
+            return None
 
         add_late(residual, finish)
+
+    def forward_rows(self, x, batch, entry):
+        """The mixer's output alone: the output projection's float32 sums and its bias."""
+        out = L.linear(self._heads(x, batch, entry), self.wo, out_dtype=torch.float32)
+        return out if self.bo is None else K.add_bias(out, self.bo)
 
 
 register_mixer("mixed_heads_attention", MixedHeadsAttention)

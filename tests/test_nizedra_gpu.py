@@ -599,7 +599,7 @@ def test_trace_replay_program(tmp_path):
 
     import numpy as np
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    folder = make_folder(tmp_path, "A", seed=19)
+    folder = make_folder(tmp_path, "C", seed=19)
     cfg, w = P.load_folder(folder)
     V = cfg["vocab"]
     reqs = {"a": util.random_tokens(V, 150, 1), "b": util.random_tokens(V, 9, 2), "c": util.random_tokens(V, 1, 3),
