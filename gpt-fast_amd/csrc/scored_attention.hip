@@ -278,6 +278,18 @@ union SAFrag {
 };
 
 #define SA_SROW 36            // floats per row of a wave's score tile in shared memory (32 + 4)
+#define SA_LUT_MAX 8192       // distances whose rows a workgroup with a mix keeps in shared memory
+
+// floats of shared memory before the score tiles of a workgroup with a mix: talk [H][H], the
+// distance table [rows][H] and, if it is short enough, the distances' rows
+__host__ __device__ inline int sam_tables(int H, int bias_rows, int n_lookup, bool with_bias) {
+    int n = (H * H + 3) / 4 * 4;
+    if (with_bias) {
+        n += (bias_rows * H + 3) / 4 * 4;
+        if (n_lookup <= SA_LUT_MAX) n += (n_lookup + 3) / 4 * 4;
+    }
+    return n;
+}
 
 __device__ __forceinline__ float sa_max_lane_groups(float v) {
     v = fmaxf(v, __shfl_xor(v, 16, GFA_WAVE));
@@ -348,10 +360,24 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
     const int lo_min = (s.window > 0 && spos + tok_lo - s.window + 1 > 0) ? spos + tok_lo - s.window + 1 : 0;
     const int last_key = spos + q_len - 1;             // the newest key the cache holds of this sequence
 
-    float* talk_lds = sam_lds;                         // [H][H], with a mix
-    float* tiles = sam_lds + (mix ? s.H * s.H : 0);    // [waves][16][SA_SROW]
+    // with a mix the small tables live in shared memory (the workgroup walks many key blocks
+    // and reads them at every one)
+    float* talk_lds = sam_lds;                         // [H][H]
+    float* tiles = sam_lds + (mix ? sam_tables(s.H, s.bias_rows, s.n_lookup, bias != nullptr) : 0);
+    const float* bias_t = bias;                        // [rows][H]
+    const int* lookup_t = lookup;
     if (mix) {
         for (int e = threadIdx.x; e < s.H * s.H; e += blockDim.x) talk_lds[e] = talk[e];
+        if (bias) {
+            float* b_lds = sam_lds + (s.H * s.H + 3) / 4 * 4;
+            for (int e = threadIdx.x; e < s.bias_rows * s.H; e += blockDim.x) b_lds[e] = bias[e];
+            bias_t = b_lds;
+            if (s.n_lookup <= SA_LUT_MAX) {
+                int* l_lds = (int*)(b_lds + (s.bias_rows * s.H + 3) / 4 * 4);
+                for (int e = threadIdx.x; e < s.n_lookup; e += blockDim.x) l_lds[e] = lookup[e];
+                lookup_t = l_lds;
+            }
+        }
         __syncthreads();
     }
 
@@ -374,6 +400,15 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
         const int page = pages[bi >> 1];
         const bf16_t* kb = k_pages + cache_region(page, g, s.G, s.hd) + (size_t)(bi & 1) * 32 * s.hd;
         const bf16_t* vb = v_pages + cache_region(page, g, s.G, s.vd) + (size_t)(bi & 1) * 512;
+        // few value tiles: their loads are asked for with the keys', ahead of the scores' work
+        SAFrag vpre[DVT <= 8 ? DVT : 1];
+        if (DVT <= 8) {
+#pragma unroll
+            for (int dt = 0; dt < (DVT <= 8 ? DVT : 1); ++dt) {
+                const int dtc = dt < vtiles ? dt : vtiles - 1;
+                vpre[dt].u = *(const uint4*)(vb + (size_t)dtc * 1024 + lg * 128 + li * 8);
+            }
+        }
         sa_floatx4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kk = 0; kk < DK; ++kk) {
@@ -395,8 +430,8 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
             if (s.softcap > 0.f) v = s.softcap * tanhf(v / s.softcap);
             if (bias && j <= pos) {
                 const int dist = pos - j;
-                const int row = dist < s.n_lookup ? lookup[dist] : s.bias_rows - 1;
-                v += bias[(size_t)row * s.H + head];
+                const int row = dist < s.n_lookup ? lookup_t[dist] : s.bias_rows - 1;
+                v += bias_t[(size_t)row * s.H + head];
             }
             // what lies beyond the newest key may be anything: it must not reach the mix
             sv[e] = j <= last_key ? v : 0.f;
@@ -457,7 +492,8 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
         for (int dt = 0; dt < DVT; ++dt) {
             const int dtc = dt < vtiles ? dt : vtiles - 1;
             SAFrag vf;
-            vf.u = *(const uint4*)(vb + (size_t)dtc * 1024 + lg * 128 + li * 8);
+            if (DVT <= 8) vf.u = vpre[DVT <= 8 ? dt : 0].u;
+            else vf.u = *(const uint4*)(vb + (size_t)dtc * 1024 + lg * 128 + li * 8);
             vf.u.x &= keep.x;
             vf.u.y &= keep.y;
             vf.u.z &= keep.z;
@@ -530,8 +566,18 @@ static int sam_launch(const void* q, const void* k_pages, const void* v_pages, c
         if (waves * 64 > MAXT) return (int)hipErrorInvalidValue;
         grid = dim3((max_q_len + tp - 1) / tp, 1, n_seqs);
         block = dim3(waves * 64);
-        shmem = sizeof(float) * ((size_t)s.H * s.H + (size_t)waves * 16 * SA_SROW);
-        if (shmem > 64 * 1024) return (int)hipErrorInvalidValue;
+        shmem = sizeof(float) * ((size_t)sam_tables(s.H, s.bias_rows, s.n_lookup, bias != nullptr)
+                                 + (size_t)waves * 16 * SA_SROW);
+        if (shmem > 64 * 1024) {
+            static bool allowed = false;
+            if (!allowed) {
+                const hipError_t e = hipFuncSetAttribute(
+                    (const void*)scored_attention_mfma_kernel<DK, DVT, MAXT, SPLIT>,
+                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return (int)e;
+                allowed = true;
+            }
+        }
     } else if (SPLIT) {
         // as many waves as their partial results fit the shared memory a workgroup may have
         const int waves = s.vd > 256 ? 4 : 8;
@@ -567,7 +613,9 @@ extern "C" int gfa_scored_attention_mfma_takes(int H, int G, int hd, int vd, int
         if (H > 64 || (gs <= 16 && 16 / gs < 1)) return 0;
         const bool small = hd <= 128 && vd <= 128;
         if (waves > (small ? 16 : 4)) return 0;
-        if (sizeof(float) * ((size_t)H * H + (size_t)waves * 16 * SA_SROW) > 64 * 1024) return 0;
+        // talk, a distance table of up to 64 rows and its distances' rows, the tiles
+        if (sizeof(float) * ((size_t)H * H + 64 * H + SA_LUT_MAX + 16 + (size_t)waves * 16 * SA_SROW)
+                > 150 * 1024) return 0;
     }
     return 1;
 }
