@@ -641,7 +641,7 @@ extern "C" int gfa_scored_attention_mfma(const void* q, const void* k_pages, con
     if (max_q_len == 1 && talk == nullptr) {
         if (hd <= 128 && vd <= 128) SAM_GO(4, 8, 512, true);
         if (hd <= 256 && vd <= 256) SAM_GO(8, 16, 512, true);
-        SAM_GO(18, 32, 512, true);
+        SAM_GO(18, 32, 256, true);               // four waves: a wave per SIMD has its 512 registers
     }
     if (hd <= 128 && vd <= 128) SAM_GO(4, 8, 1024, false);
     if (hd <= 256 && vd <= 256) SAM_GO(8, 16, 256, false);
