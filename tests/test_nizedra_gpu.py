@@ -139,6 +139,172 @@ def test_distance_rows_of_the_bias_table():
         assert all(x <= y for x, y in zip(table, table[1:]))
 
 
+def _table_and_positions(lens, starts):
+    """Pages handed out in reverse; the step's token maps."""
+    total = [s + l for s, l in zip(starts, lens)]
+    n_pages = sum((t + 63) // 64 for t in total)
+    order, tables, at = list(range(n_pages))[::-1], [], 0
+    for t in total:
+        n = (t + 63) // 64
+        tables.append(order[at:at + n])
+        at += n
+    widest = max(len(t) for t in tables)
+    table = torch.tensor([t + [-1] * (widest - len(t)) for t in tables], dtype=torch.int32, device=DEV)
+    tok_seq = torch.tensor([b for b, l in enumerate(lens) for _ in range(l)], dtype=torch.int32, device=DEV)
+    pos = [s + i for s, l in zip(starts, lens) for i in range(l)]
+    return n_pages, tables, table, tok_seq, torch.tensor(pos, dtype=torch.int32, device=DEV), pos
+
+
+def _cache_rows(k_pages, v_pages, d, dv):
+    """What the kernels keep -> keys [n, G, 64, d] and values [n, G, dv, 64]."""
+    n, G = k_pages.shape[:2]
+    k = k_pages.reshape(n, G, -1)[..., util.key_places(d).reshape(-1)].view(n, G, 64, d)
+    v = v_pages.reshape(n, G, -1)[..., util.value_places(dv).reshape(-1)].view(n, G, dv, 64)
+    return k.double().cpu(), v.double().cpu()
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("H,G,d,dv,eps", [(4, 2, 16, 16, 1e-5), (3, 3, 20, 12, 1e-3), (6, 1, 8, 24, None), (2, 1, 10, 6, 1e-6)])
+def test_unit_norm_heads_and_their_place_in_the_cache(dtype, tol, H, G, d, dv, eps):
+    from gpt_fast_amd.ops import scored_attention as SA
+    torch.manual_seed(H + d)
+    lens, starts = [70, 1, 3], [0, 130, 62]
+    n_pages, tables, table, tok_seq, tok_pos, pos = _table_and_positions(lens, starts)
+    width = (H + G) * d + G * dv
+    proj = torch.randn(sum(lens), width + 3, device=DEV) * 2          # rows wider than what is read
+    bias = torch.randn(width, device=DEV)
+    k_pages = torch.zeros(n_pages, G, 64, d, device=DEV, dtype=dtype)
+    v_pages = torch.zeros(n_pages, G, dv, 64, device=DEV, dtype=dtype)
+    q = SA.unit_heads_store(proj, bias, tok_seq, tok_pos, table, k_pages, v_pages, H, G, d, dv, eps, dtype)
+    x = proj[:, :width].double().cpu() + bias.double().cpu()
+    unit = (lambda t: t) if eps is None else (lambda t: P.unit_rms(t, eps))
+    want_q = unit(x[:, :H * d].view(-1, H, d))
+    want_k = unit(x[:, H * d:(H + G) * d].view(-1, G, d))
+    want_v = x[:, (H + G) * d:].view(-1, G, dv)
+    assert rel_err(q, want_q) < tol
+    k, v = _cache_rows(k_pages, v_pages, d, dv)
+    seqs = [b for b, l in enumerate(lens) for _ in range(l)]
+    for n, (b, p_) in enumerate(zip(seqs, pos)):
+        page = tables[b][p_ // 64]
+        assert rel_err(k[page, :, p_ % 64], want_k[n]) < tol
+        assert rel_err(v[page, :, :, p_ % 64], want_v[n]) < tol
+    # without pages nothing is stored and q is the same
+    q2 = SA.unit_heads_store(proj, bias, tok_seq, tok_pos, table, None, None, H, G, d, dv, eps, dtype)
+    assert torch.equal(q, q2)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
+@pytest.mark.parametrize("H,d,dr,R,Q,rot", [(3, 16, 8, 32, 40, 8), (2, 12, 8, 20, 28, 4), (4, 8, 16, 144, 24, 16),
+                                          (2, 10, 6, 10, 14, 2), (2, 8, 4, 16, 8, 0)])
+def test_latents_their_norms_rotation_and_place_in_the_cache(dtype, tol, H, d, dr, R, Q, rot):
+    from gpt_fast_amd.ops import scored_attention as SA
+    from gpt_fast_amd.parts.position import rotary_frequencies
+    torch.manual_seed(R + Q)
+    lens, starts = [70, 1, 3], [0, 130, 62]
+    n_pages, tables, table, tok_seq, tok_pos, pos = _table_and_positions(lens, starts)
+    N = sum(lens)
+    proj = torch.randn(N, Q + R + dr + 5, device=DEV) * 2
+    wq, wkv = 1 + 0.3 * torch.randn(Q, device=DEV), 1 + 0.3 * torch.randn(R, device=DEV)
+    freqs = rotary_frequencies(rot, 777.0).to(DEV) if rot else None
+    k_pages = torch.zeros(n_pages, 1, 64, R + dr, device=DEV, dtype=dtype)
+    v_pages = torch.zeros(n_pages, 1, R, 64, device=DEV, dtype=dtype)
+    cq = SA.latent_store(proj, Q, R, dr, wq, wkv, 1e-4, freqs, rot, tok_seq, tok_pos, table, k_pages, v_pages, dtype)
+    x = proj.double().cpu()
+    positions = torch.tensor(pos)
+    assert rel_err(cq, P.rms_norm(x[:, :Q], wq.double().cpu(), 1e-4)) < tol
+    want_c = P.rms_norm(x[:, Q:Q + R], wkv.double().cpu(), 1e-4)
+    want_kr = P.rotate_pairs(x[:, Q + R:Q + R + dr], positions, rot, 777.0)
+    k, v = _cache_rows(k_pages, v_pages, R + dr, R)
+    seqs = [b for b, l in enumerate(lens) for _ in range(l)]
+    for n, (b, p_) in enumerate(zip(seqs, pos)):
+        page = tables[b][p_ // 64]
+        assert rel_err(k[page, 0, p_ % 64, :R], want_c[n]) < tol
+        assert rel_err(k[page, 0, p_ % 64, R:], want_kr[n]) < tol
+        assert rel_err(v[page, 0, :, p_ % 64], want_c[n]) < tol
+    # the query: plain parts head by head, rotated parts behind the room for the latent's part
+    q = torch.randn(N, H * (d + dr), device=DEV)
+    plain, full = SA.latent_query(q, freqs, rot, tok_pos, H, d, dr, R, dtype)
+    qq = q.double().cpu().view(N, H, d + dr)
+    assert rel_err(plain.permute(1, 0, 2), qq[..., :d]) < tol
+    assert rel_err(full.permute(1, 0, 2)[..., R:], P.rotate_pairs(qq[..., d:], positions, rot, 777.0)) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-5), ("bfloat16", 2e-2)])
+def test_parts_alone_the_input_mix_the_dense_feed_forward_and_the_sandwich_block(dtype, tol):
+    from gpt_fast_amd.config.spec import (DenseFeedForwardSpec, InputMixSpec, LayerSpec, NormSpec)
+    from gpt_fast_amd.parts.base import BLOCKS, FEED_FORWARDS, STREAM_STEPS, Runtime
+    from gpt_fast_amd.parts.model import _Arranged
+    import gpt_fast_amd as gfa
+    rt = Runtime(torch.float32 if dtype == "float32" else torch.bfloat16, DEV)
+    torch.manual_seed(5)
+    for rows in (1, 5, 40, 150):
+        D, F_ = 72, 136
+        mix = STREAM_STEPS.build(InputMixSpec(D, "loop.w"), rt)
+        w = (torch.randn(D, 2 * D, device=DEV) * 0.2).to(rt.dtype)
+        mix.bind({"loop.w": w})
+        x, x0 = torch.randn(rows, D, device=DEV), torch.randn(rows, D, device=DEV)
+        want = torch.cat([x, x0], 1).double().cpu() @ w.double().cpu().T
+        got = mix.forward(x, x0, None)
+        assert got.dtype == torch.float32 and rel_err(got, want) < tol
+
+        ff = FEED_FORWARDS.build(DenseFeedForwardSpec(D, F_, "xielu"), rt)
+        up = (torch.randn(F_, D, device=DEV) * 0.3).to(rt.dtype)
+        down = (torch.randn(D, F_, device=DEV) * 0.3).to(rt.dtype)
+        act = torch.tensor([0.4, -0.9], device=DEV)
+        ff.bind({"w_up": up, "w_down": down, "act": act})
+        h = torch.randn(rows, D, device=DEV).to(rt.dtype)
+        want = P.dense_feed_forward(h.double().cpu(), up.double().cpu(), down.double().cpu(), act.double().cpu())
+        assert rel_err(ff.forward_rows(h, None), want) < tol
+        res = torch.randn(rows, D, device=DEV)
+        before = res.double().cpu()
+        ff.forward(h, None, res)
+        assert rel_err(res.double().cpu() - before, want) < max(tol, 1e-4)
+
+    # the block: x + n1b(mixer(n1(x))), then + n2b(ff(n2(.))), with a toy mixer that doubles its input
+    class Doubling:
+        kind = "doubling_for_a_test"
+    class DoublingMixer:
+        def __init__(self, spec, runtime):
+            pass
+        def parameters(self):
+            return {}
+        def bind(self, tensors):
+            pass
+        def cache_need(self):
+            return None
+        def forward(self, x, batch, entry, residual):
+            residual += 2.0 * x.float()
+    gfa.register_mixer("doubling_for_a_test", DoublingMixer)
+    D, F_ = 40, 64
+    norm = lambda: NormSpec(D, 1e-5)
+    layer = LayerSpec(name="l", arrangement="sandwich_norm", mixer=Doubling(), mixer_norm=norm(),
+                      mixer_out_norm=norm(), feed_forward=DenseFeedForwardSpec(D, F_, "xielu"),
+                      feed_forward_norm=norm(), feed_forward_out_norm=norm())
+    block = BLOCKS.build(_Arranged(layer), rt)
+    names = sorted(block.parameters())
+    assert names == ["feed_forward.act", "feed_forward.w_down", "feed_forward.w_up", "feed_forward_norm.weight",
+                     "feed_forward_out_norm.weight", "mixer_norm.weight", "mixer_out_norm.weight"]
+    t = {n: (1 + 0.3 * torch.randn(D, device=DEV)) for n in names if n.endswith("weight")}
+    t["feed_forward.w_up"] = (torch.randn(F_, D, device=DEV) * 0.3).to(rt.dtype)
+    t["feed_forward.w_down"] = (torch.randn(D, F_, device=DEV) * 0.3).to(rt.dtype)
+    t["feed_forward.act"] = torch.tensor([0.1, 0.2], device=DEV)
+    block.bind(t)
+    for rows in (3, 50):
+        x = torch.randn(rows, D, device=DEV)
+        res = x.clone()
+        block.forward(res, None, None)
+        d = {k: v.double().cpu() for k, v in t.items()}
+        xx = x.double().cpu()
+        n1 = P.rms_norm(xx, d["mixer_norm.weight"], 1e-5)
+        if dtype == "bfloat16":
+            n1 = n1.bfloat16().double()
+        hh = xx + P.rms_norm(2 * n1, d["mixer_out_norm.weight"], 1e-5)
+        y = P.dense_feed_forward(P.rms_norm(hh, d["feed_forward_norm.weight"], 1e-5), d["feed_forward.w_up"],
+                                 d["feed_forward.w_down"], d["feed_forward.act"])
+        want = hh + P.rms_norm(y, d["feed_forward_out_norm.weight"], 1e-5)
+        assert rel_err(res, want) < tol
+
+
 @pytest.mark.parametrize("H,dk,dv", [(2, 16, 32), (1, 24, 40), (3, 20, 12), (2, 72, 8), (1, 130, 33),
                                      (3, 10, 6), (2, 128, 128), (2, 64, 16)])
 @pytest.mark.parametrize("chunked", [False, True])
