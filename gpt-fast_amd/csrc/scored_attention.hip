@@ -643,7 +643,18 @@ extern "C" int gfa_scored_attention_mfma(const void* q, const void* k_pages, con
         if (hd <= 256 && vd <= 256) SAM_GO(8, 16, 512, true);
         SAM_GO(18, 32, 256, true);               // four waves: a wave per SIMD has its 512 registers
     }
-    if (hd <= 128 && vd <= 128) SAM_GO(4, 8, 1024, false);
+    if (hd <= 128 && vd <= 128) {
+        // the workgroup's size bounds a wave's registers: no larger than the waves of a mix need
+        const int gs = H / G;
+        const int waves = talk ? G * (gs > 16 ? (gs + 15) / 16 : 1) : 4;
+        // (a prompt's many workgroups of eight waves run faster two to a compute unit with 128
+        // registers a wave and a few of them in scratch memory - 660 against 748 us for 2,048
+        // tokens of 32 heads - than one to a compute unit with all in registers; single-token
+        // steps the other way round)
+        if (waves <= 4) SAM_GO(4, 8, 256, false);
+        if (waves <= 8 && max_q_len <= 16) SAM_GO(4, 8, 512, false);
+        SAM_GO(4, 8, 1024, false);
+    }
     if (hd <= 256 && vd <= 256) SAM_GO(8, 16, 256, false);
     SAM_GO(18, 32, 256, false);
 #undef SAM_GO
