@@ -389,6 +389,7 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
         qf[kk].u = d < s.hd ? *(const uint4*)(qrow + d) : make_uint4(0, 0, 0, 0);
     }
     const float row_scale = s.scale * (temperature ? temperature[head] : 1.f);
+    const float cap_exp = s.softcap > 0.f ? 2.885390081777927f / s.softcap : 0.f;     // 2 log2(e) / cap
     const int vtiles = s.vd / 16;
     sa_floatx4_t o[DVT];
 #pragma unroll
@@ -427,7 +428,9 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
         for (int e = 0; e < 8; ++e) {
             const int j = key0 + e;
             float v = sv[e] * row_scale;
-            if (s.softcap > 0.f) v = s.softcap * tanhf(v / s.softcap);
+            // cap tanh(v / cap) = cap (1 - 2 / (e^(2 v / cap) + 1)): one exponential and one
+            // reciprocal; exact at both ends, within a few 1e-7 of cap elsewhere
+            if (s.softcap > 0.f) v = s.softcap - 2.f * s.softcap * __frcp_rn(exp2f(v * cap_exp) + 1.f);
             if (bias && j <= pos) {
                 const int dist = pos - j;
                 const int row = dist < s.n_lookup ? lookup_t[dist] : s.bias_rows - 1;
@@ -445,18 +448,22 @@ __global__ __launch_bounds__(MAXT) void scored_attention_mfma_kernel(
             const float* trow = talk_lds + head * s.H;
             // first row of this lane's token in a tile
             const int tok_row = (gs > 16 || !row_ok) ? 0 : (li / gs) * gs;
+            // head h2 = g2 gs + r2 of this lane's token is row g2 tpg 16 + tok_row + r2 of the tiles
             const int tpg = gs > 16 ? (gs + 15) / 16 : 1;
-            for (int h2 = 0; h2 < s.H; ++h2) {
-                const int g2 = h2 / gs, r2 = h2 - g2 * gs;
-                const int w2 = g2 * tpg + (r2 >> 4);
-                const int row2 = gs > 16 ? (r2 & 15) : tok_row + r2;
-                const float* src = tiles + ((size_t)w2 * 16 + row2) * SA_SROW + lg * 8;
-                const float4 a = *(const float4*)src, b = *(const float4*)(src + 4);
-                const float t = trow[h2];
-                z[0] = fmaf(t, a.x, z[0]); z[1] = fmaf(t, a.y, z[1]);
-                z[2] = fmaf(t, a.z, z[2]); z[3] = fmaf(t, a.w, z[3]);
-                z[4] = fmaf(t, b.x, z[4]); z[5] = fmaf(t, b.y, z[5]);
-                z[6] = fmaf(t, b.z, z[6]); z[7] = fmaf(t, b.w, z[7]);
+            const float* tile_row = tiles + (size_t)tok_row * SA_SROW + lg * 8;
+            for (int g2 = 0; g2 < s.G; ++g2) {
+                const float* src = tile_row + (size_t)g2 * tpg * 16 * SA_SROW;
+                const float* tg = trow + g2 * gs;
+#pragma unroll 4
+                for (int r2 = 0; r2 < gs; ++r2) {
+                    const float4 a = *(const float4*)src, b = *(const float4*)(src + 4);
+                    const float t = tg[r2];
+                    z[0] = fmaf(t, a.x, z[0]); z[1] = fmaf(t, a.y, z[1]);
+                    z[2] = fmaf(t, a.z, z[2]); z[3] = fmaf(t, a.w, z[3]);
+                    z[4] = fmaf(t, b.x, z[4]); z[5] = fmaf(t, b.y, z[5]);
+                    z[6] = fmaf(t, b.z, z[6]); z[7] = fmaf(t, b.w, z[7]);
+                    src += SA_SROW;
+                }
             }
 #pragma unroll
             for (int e = 0; e < 8; ++e) sv[e] = z[e];
