@@ -21,6 +21,8 @@ A step can only be recorded if every part issues the same kernels whatever the b
 holds; a part says so with ``replayable = True``.  A model with a part that does not
 (one that loops over the batch on the host, say) is stepped without a recording.
 """
+import gc
+import weakref
 from collections import OrderedDict
 from typing import List, Optional, Sequence
 
@@ -72,7 +74,9 @@ class RecordedSteps:
     there are more than ``limit`` (each holds the memory of its step's intermediates)."""
 
     def __init__(self, engine, limit: int = 8):
-        self.engine = engine
+        # no cycle with the engine that owns this: an engine nobody holds any more goes at once,
+        # with its recordings, and not whenever the collector of cycles next runs
+        self._engine = weakref.ref(engine)
         self.limit = limit
         self._steps: "OrderedDict[tuple, RecordedStep]" = OrderedDict()
 
@@ -83,7 +87,7 @@ class RecordedSteps:
             self._steps.move_to_end(key)
         else:
             # none of this shape, or it is in use by another open session
-            step = RecordedStep(self.engine, n_rows, widths, params)
+            step = RecordedStep(self._engine(), n_rows, widths, params)
             if key not in self._steps:
                 self._steps[key] = step
                 for old in [k for k, s in self._steps.items() if not s.busy and k != key]:
@@ -209,8 +213,20 @@ class DecodeSession:
         for restore in put_back:
             restore()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            self._run()
+        # Nothing may be destroyed while the step is recorded: a dead cycle of Python objects
+        # that holds another recording, pinned buffers or events, collected in the middle of
+        # the capture, ends the process (torch's graph context no longer collects garbage
+        # before it starts).  So the collector runs now and is held off until the recording is
+        # done.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                self._run()
+        finally:
+            if collecting:
+                gc.enable()
         self.rec.graph = graph
 
     @torch.no_grad()
