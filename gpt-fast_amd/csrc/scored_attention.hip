@@ -201,7 +201,16 @@ static int sa_launch(const void* q, const void* k_pages, const void* v_pages, co
                      int n_tokens, const SAShape& s, hipStream_t stream) {
     constexpr int HB = SA_WAVES * HPW;
     const size_t shmem = (size_t)HB * (s.hd + 2 * GFA_PAGE) * sizeof(float);
-    if (shmem > 64 * 1024) return (int)hipErrorInvalidValue;
+    if (shmem > 160 * 1024) return (int)hipErrorInvalidValue;
+    if (shmem > 64 * 1024) {
+        static bool allowed = false;
+        if (!allowed) {
+            const hipError_t e = hipFuncSetAttribute((const void*)scored_attention_kernel<T, HPW, VPT>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return (int)e;
+            allowed = true;
+        }
+    }
     dim3 grid(n_tokens, (s.H + HB - 1) / HB);
     scored_attention_kernel<T, HPW, VPT><<<grid, SA_THREADS, shmem, stream>>>(
         (const T*)q, (const T*)k_pages, (const T*)v_pages, tok_seq, tok_pos, table, temperature,
@@ -227,6 +236,7 @@ static int sa_dispatch(const void* q, const void* k_pages, const void* v_pages, 
         if (vpt <= 8) SA_GO(4, 8);
     } else if (hpw <= 16) {
         if (vpt <= 2) SA_GO(16, 2);
+        if (vpt <= 8) SA_GO(16, 8);
     }
 #undef SA_GO
     return (int)hipErrorInvalidValue;
@@ -587,8 +597,8 @@ static int sam_launch(const void* q, const void* k_pages, const void* v_pages, c
         }
     } else if (SPLIT) {
         // as many waves as their partial results fit the shared memory a workgroup may have
-        const int waves = s.vd > 256 ? 4 : 8;
-        if (waves * 64 > MAXT) return (int)hipErrorInvalidValue;
+        int waves = s.vd > 256 ? 4 : 8;
+        if (waves * 64 > MAXT) waves = MAXT / 64;      // the kernel built for fewer, with more registers
         grid = dim3((max_q_len * gs + 15) / 16, s.G, n_seqs);
         block = dim3(waves * 64);
         shmem = sizeof(float) * (size_t)waves * (32 + (size_t)s.vd * 16);

@@ -89,8 +89,8 @@ def attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tok
         rows = bias.shape[0]
     if talk is not None and H > 64:
         raise KernelError("scored attention: scores are mixed across at most 64 heads")
-    if vd > 512 or (talk is not None and H > 16 and vd > 128):
-        raise KernelError(f"scored attention: value size {vd} with {H} heads is not supported")
+    if vd > 512:
+        raise KernelError(f"scored attention: value size {vd} is not supported (up to 512)")
     shape = (H, n, vd) if head_major else (n, H, vd)
     if out is None:
         out = torch.empty(shape, dtype=q.dtype, device=q.device)

@@ -452,7 +452,8 @@ def _scored_attention_alone(dtype, H, G, d, dv, window, lens, starts, mixed, hea
     (3, 1, 40, 32, 24, False, True), (2, 1, 28, 20, None, False, True), (4, 1, 160, 144, 70, False, True),
     (2, 1, 16, 10, 9, False, True), (5, 1, 576, 512, 100, False, True), (4, 2, 64, 64, 33, False, False),
     (32, 1, 16, 16, None, True, False), (6, 2, 16, 32, None, True, False), (3, 3, 24, 16, None, True, False),
-    (32, 8, 128, 128, None, True, False), (40, 1, 72, 64, 50, False, True)])
+    (32, 8, 128, 128, None, True, False), (40, 1, 72, 64, 50, False, True),
+    (16, 1, 320, 256, 300, False, True), (20, 4, 24, 144, None, True, False), (24, 2, 200, 32, None, True, False)])
 @pytest.mark.parametrize("by_sequence", [False, True])
 def test_scored_attention_alone(dtype, tol, H, G, d, dv, window, mixed, head_major, by_sequence):
     """A prompt, a portion at an offset, single tokens and a first token, in one launch; on the
@@ -465,6 +466,7 @@ def test_scored_attention_alone(dtype, tol, H, G, d, dv, window, mixed, head_maj
 
 
 @pytest.mark.parametrize("H,G,d,dv,window", [(3, 1, 40, 32, 24), (32, 1, 576, 512, 300), (4, 1, 160, 144, 70),
+                                             (16, 1, 320, 256, 300), (16, 1, 264, 128, None),
                                              (40, 1, 72, 64, None), (4, 2, 64, 64, 33), (8, 8, 128, 128, None)])
 def test_single_token_steps_share_their_key_blocks_among_waves(H, G, d, dv, window):
     """One token per sequence, no mix: sequences of one key, of less than a block, of several
