@@ -63,8 +63,9 @@ __global__ __launch_bounds__(SA_THREADS) void scored_attention_kernel(
         const float* __restrict__ talk, T* __restrict__ out, SAShape s) {
     extern __shared__ __attribute__((aligned(16))) float sa_lds[];
     constexpr int HB = SA_WAVES * HPW;
-    float* qs = sa_lds;                          // [HB][hd]
-    float* sc = qs + HB * s.hd;                  // [HB][64] scores before the mix
+    const int nh = s.H < HB ? s.H : HB;          // heads a block really has
+    float* qs = sa_lds;                          // [nh][hd]
+    float* sc = qs + nh * s.hd;                  // [HB][64] scores before the mix
     float* pr = sc + HB * GFA_PAGE;              // [HB][64] softmax weights
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = blockIdx.x, h0 = blockIdx.y * HB;
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(SA_THREADS) void scored_attention_kernel(
     const int lo = (s.window > 0 && pos - s.window + 1 > 0) ? pos - s.window + 1 : 0;
     const int per_group = s.H / s.G;
 
-    for (int e = threadIdx.x; e < HB * s.hd; e += SA_THREADS) {
+    for (int e = threadIdx.x; e < nh * s.hd; e += SA_THREADS) {
         const int hl = e / s.hd, d = e - hl * s.hd;
         qs[e] = (h0 + hl < s.H)
             ? load_as_float(q + (size_t)n * s.q_tok + (size_t)(h0 + hl) * s.q_head + d) : 0.f;
@@ -200,7 +201,7 @@ static int sa_launch(const void* q, const void* k_pages, const void* v_pages, co
                      const float* bias, const int* lookup, const float* talk, void* out,
                      int n_tokens, const SAShape& s, hipStream_t stream) {
     constexpr int HB = SA_WAVES * HPW;
-    const size_t shmem = (size_t)HB * (s.hd + 2 * GFA_PAGE) * sizeof(float);
+    const size_t shmem = ((size_t)(s.H < HB ? s.H : HB) * s.hd + (size_t)HB * 2 * GFA_PAGE) * sizeof(float);
     if (shmem > 160 * 1024) return (int)hipErrorInvalidValue;
     if (shmem > 64 * 1024) {
         static bool allowed = false;
