@@ -85,7 +85,10 @@ def nizedra_plan(c: NizedraConfig) -> ModelPlan:
 def nizedra_bindings(c: NizedraConfig) -> CheckpointLayout:
     D, V = c.width, c.vocab
     b = [Binding("embed", (Source("embed", (V, D)),))]
-    if c.loop is not None:
+    # a loop without a pass (no layer in it, or no time round) never uses its matrix: a
+    # checkpoint may still hold it
+    looped = c.loop is not None and c.loop.times > 0 and c.loop.stop > c.loop.start
+    if looped:
         b.append(Binding(LOOP_INPUT, (Source(LOOP_INPUT, (D, 2 * D)),)))
 
     def vector(target, name, shape, init="norm"):
@@ -148,7 +151,8 @@ def nizedra_bindings(c: NizedraConfig) -> CheckpointLayout:
             ]
     b.append(vector("final.norm.weight", "final.norm", (D,)))
     b.append(Binding("head", (Source("head", (V, D)),)))
-    return CheckpointLayout(tuple(b))
+    unused = (r"^loop\.in$",) if c.loop is not None and not looped else ()
+    return CheckpointLayout(tuple(b), ignored=unused)
 
 
 _REL = re.compile(r"^l(\d+)\.mix\.rel$")

@@ -105,6 +105,27 @@ def test_model_folder_tensors_and_sizes_from_their_shapes(tmp_path, name):
         load_parameters(folder, arch.layouts(arch.read_config(other)), "float32", None)
 
 
+def test_a_loop_without_a_pass_needs_no_matrix_and_tolerates_one(tmp_path):
+    import gpt_fast_amd as gfa
+    from gpt_fast_amd.weights.bindings import load_parameters
+    from gpt_fast_amd.weights.safetensors_io import write_safetensors
+    from nizedra_cases import write_model
+    for loop in ({"start": 1, "stop": 1, "times": 2}, {"start": 0, "stop": 2, "times": 0}):
+        raw = {**CASES["B"], "loop": loop}
+        folder = write_model(str(tmp_path / f"empty{loop['times']}"), raw, 3)
+        arch, cfg = gfa.read_model_folder(folder)
+        plan = arch.plan(cfg)
+        assert all(r.enter is None for r in plan.order)
+        assert [r.layer for r in plan.order] == [i for i, _ in P.run_order(raw)]
+        params = load_parameters(folder, arch.layouts(cfg), "float32", None)
+        assert "loop.in" not in params
+        # ... and with the matrix in the file
+        _, w = P.load_folder(folder)
+        w["loop.in"] = torch.zeros(raw["width"], 2 * raw["width"])
+        write_safetensors(os.path.join(folder, "model.safetensors"), {k: v.float() for k, v in w.items()})
+        assert "loop.in" not in load_parameters(folder, arch.layouts(cfg), "float32", None)
+
+
 def test_cache_entries_of_a_looped_layer_are_apart(tmp_path):
     import gpt_fast_amd as gfa
     from gpt_fast_amd.cache.store import Cache
