@@ -46,6 +46,11 @@ def linear_scaled(freqs: torch.Tensor, factor: float, **_ignored) -> torch.Tenso
 FREQUENCY_SCALINGS = {"llama3": llama3_scaled, "linear": linear_scaled}
 
 
+# the kernel that rotates, stores and attends in one (csrc/attention_bf16.hip: gfa_attention_sliced_bf16)
+# is not used: see RotaryPosition.rotate_store_attend
+FUSED_SLICED_ATTENTION = False
+
+
 class RotaryPosition(Part):
     LAYOUTS = {"interleaved": 0, "half": 1}
     replayable = True
@@ -89,7 +94,18 @@ class RotaryPosition(Part):
     def rotate_store_attend(self, qkv, batch, entry, n_heads, n_kv_heads, head_dim, scale, window):
         """For a step of one token per sequence whose ``qkv`` is still an
         ``ops.linear.SlicedRows``: rotation, cache write and attention in one kernel.  None:
-        not available for this step (the caller rotates, stores and attends apart)."""
+        not available for this step (the caller rotates, stores and attends apart).
+
+        Switched off (``FUSED_SLICED_ATTENTION``): the kernel puts the token's own key into the
+        operand registers of the block it has loaded from the cache, and in some sequences of
+        a step - other ones from run to run - what the cache held at that place reaches the
+        product instead: with the pool's never-written slots holding bytes that are no number,
+        20 sequences decoding together gave rows that are no number; with other bytes the
+        token's own score is quietly that of a stale key.  Rotating and storing apart and then
+        attending (3 us more a layer at 17..64 rows) reads the key back from the cache and does
+        not show it."""
+        if not FUSED_SLICED_ATTENTION:
+            return None
         # a run that reads another run's cache attends to that run's keys and values, also at
         # the token's own position: not to the ones this kernel would make of its own rows
         if (self.spec.layout != "interleaved" or not isinstance(qkv, L.SlicedRows)

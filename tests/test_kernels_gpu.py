@@ -734,6 +734,9 @@ def test_rope_and_cache_write_over_partial_sums(H, G, hd, rot, S):
         close(vc[page, :, :, p % 64], ref[n, H + G:], 1e-2)
 
 
+@pytest.mark.skip(reason="the kernel is switched off (parts/position.py: FUSED_SLICED_ATTENTION): in some "
+                         "sequences of a step, other ones from run to run, what the cache held at the "
+                         "token's own place reaches the product instead of the token's key")
 @pytest.mark.parametrize("window", [0, 50])
 @pytest.mark.parametrize("H,G,hd,rot,S", [(32, 8, 128, 128, 4), (6, 2, 32, 16, 3), (4, 4, 64, 64, 1),
                                           (16, 1, 16, 0, 2), (12, 3, 48, 24, 2)])
